@@ -1,0 +1,299 @@
+"""Python host-side mirror of the llm.c-style launcher surface, bound over the
+C ABI of ``libgpt2_mi355x.so`` (declared in ``include/gpt2_mi355x.h``).
+
+The launchers keep the reference's names and argument order
+(``matmul_forward(out, inp, weight, bias, B, T, C, OC)`` and so on: reference
+``kernels/matmul/2_matmul_cublas.cuh:34-42``,
+``kernels/attention/3_flash_attention_permute.cuh:346-351``,
+``kernels/fused_residual_layernorm/fused_residual_layernorm.cuh:88-90``).
+Arguments are torch CUDA tensors, used only as owners of device memory: the
+library receives raw pointers.  There is no CPU fallback: if the shared library
+is missing or no GPU is present, calls raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ROOT = os.path.dirname(_HERE)
+LIB_PATH = os.path.join(_HERE, "libgpt2_mi355x.so")
+SOURCES = ("layernorm.hip", "elementwise.hip", "matmul.hip", "attention.hip", "gpt2.hip")
+HIPCC_FLAGS = (
+    "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
+    # packed-fp32 VALU forms are switched off for every HIP translation unit
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+)
+
+EXPORTS = (
+    "gpt2hip_last_error",
+    "encoder_forward", "encoder_forward_status",
+    "layernorm_forward", "layernorm_forward_status",
+    "fused_residual_layernorm_forward", "fused_residual_layernorm_forward_status",
+    "residual_forward", "residual_forward_status",
+    "gelu_forward", "gelu_forward_status",
+    "matmul_forward", "matmul_forward_status",
+    "matmul_forward_gelu", "matmul_forward_gelu_status",
+    "attention_forward", "attention_forward_status",
+    "argmax_forward", "argmax_forward_status",
+    "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
+    "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
+    "gpt2_forward_device_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
+    "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
+    "gpt2hip_timer_stop_ms",
+)
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every HIP source for gfx950 into ``libgpt2_mi355x.so`` (in-tree)."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, "-I", os.path.join(_ROOT, "include"), "-o", LIB_PATH]
+    cmd += [os.path.join(_HERE, "csrc", s) for s in SOURCES]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
+    if verbose and err.strip():
+        print(err)
+    return LIB_PATH
+
+
+class GPT2Config(ctypes.Structure):
+    _fields_ = [("max_seq_len", ctypes.c_int), ("vocab_size", ctypes.c_int),
+                ("num_layers", ctypes.c_int), ("num_heads", ctypes.c_int),
+                ("channels", ctypes.c_int)]
+
+
+GPT2_124M = dict(max_seq_len=1024, vocab_size=50257, num_layers=12, num_heads=12, channels=768)
+GPT2_350M = dict(max_seq_len=1024, vocab_size=50257, num_layers=24, num_heads=16, channels=1024)
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded C-ABI library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
+                "(there is no CPU or PyTorch fallback for these kernels)")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, ci, cz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+        L.gpt2hip_last_error.restype = ctypes.c_char_p
+        sig = {
+            "encoder_forward": [vp] * 4 + [ci] * 3,
+            "layernorm_forward": [vp] * 6 + [ci] * 3,
+            "fused_residual_layernorm_forward": [vp] * 8 + [ci] * 3,
+            "residual_forward": [vp] * 3 + [ci],
+            "gelu_forward": [vp] * 2 + [ci],
+            "matmul_forward": [vp] * 4 + [ci] * 4,
+            "matmul_forward_gelu": [vp] * 4 + [ci] * 5,
+            "attention_forward": [vp] * 4 + [ci] * 4,
+            "argmax_forward": [vp] * 2 + [ci] * 2,
+        }
+        for name, args in sig.items():
+            f = getattr(L, name)
+            f.argtypes, f.restype = args, None
+            f = getattr(L, name + "_status")
+            f.argtypes, f.restype = args, ci
+        L.gpt2_create.argtypes, L.gpt2_create.restype = [ctypes.POINTER(GPT2Config)], vp
+        L.gpt2_destroy.argtypes, L.gpt2_destroy.restype = [vp], None
+        L.gpt2_num_parameters.argtypes, L.gpt2_num_parameters.restype = [vp], cz
+        L.gpt2_params_device.argtypes, L.gpt2_params_device.restype = [vp], vp
+        L.gpt2_load_params_host.argtypes, L.gpt2_load_params_host.restype = [vp, vp, cz], ci
+        L.gpt2_reserve.argtypes, L.gpt2_reserve.restype = [vp, ci, ci], ci
+        L.gpt2_forward.argtypes, L.gpt2_forward.restype = [vp, vp, ci, ci], None
+        L.gpt2_forward_status.argtypes, L.gpt2_forward_status.restype = [vp, vp, ci, ci], ci
+        L.gpt2_forward_device_status.argtypes = [vp, vp, ci, ci]
+        L.gpt2_forward_device_status.restype = ci
+        L.gpt2_logits.argtypes, L.gpt2_logits.restype = [vp], vp
+        L.gpt2_lnf.argtypes, L.gpt2_lnf.restype = [vp], vp
+        L.gpt2_argmax_status.argtypes, L.gpt2_argmax_status.restype = [vp, vp], ci
+        L.gpt2hip_timer_create.argtypes, L.gpt2hip_timer_create.restype = [], vp
+        L.gpt2hip_timer_destroy.argtypes, L.gpt2hip_timer_destroy.restype = [vp], None
+        L.gpt2hip_timer_start.argtypes, L.gpt2hip_timer_start.restype = [vp], ci
+        L.gpt2hip_timer_stop_ms.argtypes, L.gpt2hip_timer_stop_ms.restype = [vp], ctypes.c_float
+        _lib = L
+    return _lib
+
+
+class GPT2HipError(RuntimeError):
+    pass
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().gpt2hip_last_error().decode(errors="replace")
+        raise GPT2HipError(f"{what} failed (code {rc}): {msg}")
+
+
+def _ptr(t, dtype=None) -> Optional[int]:
+    """Device pointer of a contiguous CUDA tensor (None passes NULL)."""
+    if t is None:
+        return None
+    import torch
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError("expected a CUDA tensor: these launchers take device memory only")
+    if not t.is_contiguous():
+        raise ValueError("tensor must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"expected {dtype}, got {t.dtype}")
+    return t.data_ptr()
+
+
+def _f32(t):
+    import torch
+    return _ptr(t, torch.float32)
+
+
+def _i32(t):
+    import torch
+    return _ptr(t, torch.int32)
+
+
+# ---- launchers: same names, argument order and meaning as the reference's ----
+
+def encoder_forward(out, inp, wte, wpe, B, T, C):
+    _check(lib().encoder_forward_status(_f32(out), _i32(inp), _f32(wte), _f32(wpe), B, T, C),
+           "encoder_forward")
+
+
+def layernorm_forward(out, mean, rstd, inp, weight, bias, B, T, C):
+    _check(lib().layernorm_forward_status(_f32(out), _f32(mean), _f32(rstd), _f32(inp),
+                                          _f32(weight), _f32(bias), B, T, C), "layernorm_forward")
+
+
+def fused_residual_layernorm_forward(res_out, layernorm_out, mean, rstd, inp1, inp2, weight, bias,
+                                     B, T, C):
+    _check(lib().fused_residual_layernorm_forward_status(
+        _f32(res_out), _f32(layernorm_out), _f32(mean), _f32(rstd), _f32(inp1), _f32(inp2),
+        _f32(weight), _f32(bias), B, T, C), "fused_residual_layernorm_forward")
+
+
+def residual_forward(out, inp1, inp2, N):
+    _check(lib().residual_forward_status(_f32(out), _f32(inp1), _f32(inp2), N), "residual_forward")
+
+
+def gelu_forward(out, inp, N):
+    _check(lib().gelu_forward_status(_f32(out), _f32(inp), N), "gelu_forward")
+
+
+def matmul_forward(out, inp, weight, bias, B, T, C, OC):
+    _check(lib().matmul_forward_status(_f32(out), _f32(inp), _f32(weight), _f32(bias), B, T, C,
+                                       OC), "matmul_forward")
+
+
+def matmul_forward_gelu(out, inp, weight, bias, B, T, C, OC, is_gelu):
+    _check(lib().matmul_forward_gelu_status(_f32(out), _f32(inp), _f32(weight), _f32(bias), B, T,
+                                            C, OC, int(bool(is_gelu))), "matmul_forward_gelu")
+
+
+def attention_forward(out, qkvr, att, inp, B, T, C, NH):
+    _check(lib().attention_forward_status(_f32(out), _f32(qkvr), _f32(att), _f32(inp), B, T, C,
+                                          NH), "attention_forward")
+
+
+def argmax_forward(ids, logits, N, V):
+    _check(lib().argmax_forward_status(_i32(ids), _f32(logits), N, V), "argmax_forward")
+
+
+class Timer:
+    """HIP-event timer on the null stream, the stream every launcher uses."""
+
+    def __init__(self):
+        self._h = lib().gpt2hip_timer_create()
+        if not self._h:
+            raise GPT2HipError("gpt2hip_timer_create failed")
+
+    def start(self):
+        _check(lib().gpt2hip_timer_start(self._h), "gpt2hip_timer_start")
+
+    def stop_ms(self) -> float:
+        ms = lib().gpt2hip_timer_stop_ms(self._h)
+        if ms < 0:
+            raise GPT2HipError("gpt2hip_timer_stop_ms failed")
+        return float(ms)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().gpt2hip_timer_destroy(self._h)
+            self._h = None
+
+
+class GPT2:
+    """The gpt2_forward driver (C++ side owns parameters and activations)."""
+
+    def __init__(self, *, max_seq_len, vocab_size, num_layers, num_heads, channels):
+        self.config = GPT2Config(max_seq_len, vocab_size, num_layers, num_heads, channels)
+        self._h = lib().gpt2_create(ctypes.byref(self.config))
+        if not self._h:
+            raise GPT2HipError("gpt2_create failed: " + lib().gpt2hip_last_error().decode())
+        self.num_parameters = int(lib().gpt2_num_parameters(self._h))
+        self._shape = None
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().gpt2_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def load_params(self, host_params):
+        """host_params: contiguous float32 numpy array in checkpoint order."""
+        import numpy as np
+        a = np.ascontiguousarray(host_params, dtype=np.float32)
+        _check(lib().gpt2_load_params_host(self._h, a.ctypes.data, a.size), "gpt2_load_params_host")
+
+    def params_tensor(self):
+        """A torch view of the flat device parameter buffer (no copy)."""
+        return _device_view(lib().gpt2_params_device(self._h), (self.num_parameters,), "float32")
+
+    def reserve(self, B, T):
+        _check(lib().gpt2_reserve(self._h, B, T), "gpt2_reserve")
+
+    def forward(self, inputs):
+        """inputs: (B,T) int32, numpy (host, llm.c style) or CUDA tensor (device)."""
+        import numpy as np
+        B, T = inputs.shape
+        if isinstance(inputs, np.ndarray):
+            a = np.ascontiguousarray(inputs, dtype=np.int32)
+            _check(lib().gpt2_forward_status(self._h, a.ctypes.data, B, T), "gpt2_forward")
+        else:
+            _check(lib().gpt2_forward_device_status(self._h, _i32(inputs), B, T), "gpt2_forward")
+        self._shape = (B, T)
+
+    def logits(self):
+        B, T = self._shape
+        return _device_view(lib().gpt2_logits(self._h), (B, T, self.config.vocab_size), "float32")
+
+    def lnf(self):
+        B, T = self._shape
+        return _device_view(lib().gpt2_lnf(self._h), (B, T, self.config.channels), "float32")
+
+    def argmax(self):
+        import torch
+        B, T = self._shape
+        ids = torch.empty((B, T), dtype=torch.int32, device="cuda")
+        _check(lib().gpt2_argmax_status(self._h, ids.data_ptr()), "gpt2_argmax")
+        return ids
+
+
+def _device_view(ptr: int, shape, dtype: str):
+    """Wrap library-owned device memory as a torch tensor without copying."""
+    import numpy as np
+    import torch
+
+    class _Holder:
+        pass
+
+    h = _Holder()
+    n = int(np.prod(shape))
+    h.__cuda_array_interface__ = {
+        "shape": (n,), "typestr": {"float32": "<f4", "int32": "<i4"}[dtype],
+        "data": (int(ptr), False), "version": 3, "strides": None,
+    }
+    return torch.as_tensor(h, device="cuda").view(*shape)

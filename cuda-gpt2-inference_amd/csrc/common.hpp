@@ -1,0 +1,94 @@
+// Shared host/device helpers for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+#include "gpt2_mi355x.h"
+
+namespace g2 {
+
+// ---- host-side error plumbing --------------------------------------------
+char* last_error_buffer();  // thread-local, 512 bytes (defined in capi.hip)
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(last_error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define G2_HIP(expr)                                                                       \
+  do {                                                                                     \
+    hipError_t e_ = (expr);                                                                \
+    if (e_ != hipSuccess)                                                                  \
+      return g2::fail(GPT2HIP_EHIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                      __FILE__, __LINE__);                                                 \
+  } while (0)
+
+// After a kernel launch: picks up launch-configuration errors without syncing.
+#define G2_LAUNCH_CHECK(name)                                                            \
+  do {                                                                                   \
+    hipError_t e_ = hipGetLastError();                                                   \
+    if (e_ != hipSuccess)                                                                \
+      return g2::fail(GPT2HIP_EHIP, "launch of %s failed: %s", name, hipGetErrorString(e_)); \
+  } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+[[noreturn]] inline void die(const char* what) {
+  fprintf(stderr, "[gpt2_mi355x] %s: %s\n", what, last_error_buffer());
+  abort();
+}
+
+constexpr int kWave = 64;
+
+#if defined(__HIPCC__)
+// ---- device helpers --------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Data-parallel-primitive move: value of `v` from the lane selected by CTRL.
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// All-lanes sum over a 64-wide wavefront: four DPP steps inside each row of 16
+// lanes (quad swaps, half-row mirror, row mirror), then two cross-row exchanges.
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp<0x141>(v);  // row_half_mirror
+  v += dpp<0x140>(v);  // row_mirror
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp<0xB1>(v));
+  v = fmaxf(v, dpp<0x4E>(v));
+  v = fmaxf(v, dpp<0x141>(v));
+  v = fmaxf(v, dpp<0x140>(v));
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  v = fmaxf(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+// tanh-GELU, the formula of reference 9_matmul_async_cg_tf32_gelu.cuh:5-11.
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float k = 0.7978845608028654f;  // sqrtf(2/pi)
+  const float cube = 0.044715f * x * x * x;
+  return 0.5f * x * (1.0f + tanhf(k * (x + cube)));
+}
+#endif
+
+}  // namespace g2

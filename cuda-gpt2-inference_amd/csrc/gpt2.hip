@@ -1,0 +1,269 @@
+// Host side: the gpt2_forward driver, error string and event timer.
+//
+// gpt2_forward sequences the launchers the way llm.c's train_gpt2_fp32.cu does
+// (reference README.md:9-19, images/gpt2/gpt2_flow.png), with the two fusions
+// the reference introduces: residual+layernorm in one kernel (README.md:255-268)
+// and GELU in the fc GEMM's epilogue (9_matmul_async_cg_tf32_gelu.cuh:196-212).
+// Per layer: qkv GEMM, attention, projection GEMM, fused residual+layernorm,
+// fc GEMM (+GELU), projection GEMM, fused residual+layernorm (whose layernorm
+// is the NEXT layer's ln1, or the final layernorm after the last layer).
+#include <vector>
+
+#include "common.hpp"
+
+namespace g2 {
+
+char* last_error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+enum { P_WTE, P_WPE, P_LN1W, P_LN1B, P_QKVW, P_QKVB, P_ATTPROJW, P_ATTPROJB, P_LN2W, P_LN2B,
+       P_FCW, P_FCB, P_FCPROJW, P_FCPROJB, P_LNFW, P_LNFB, P_COUNT };
+
+}  // namespace g2
+
+struct GPT2 {
+  GPT2Config cfg;
+  int device;
+  size_t num_params;
+  size_t param_off[g2::P_COUNT];
+  float* params;  // flat device buffer, checkpoint order
+
+  // activations, sized for cap_tokens = B*T
+  long long cap_tokens;
+  int* ids;        // (M)
+  float* res_a;    // (M,C) residual stream, ping
+  float* res_b;    // (M,C) residual stream, pong
+  float* ln;       // (M,C) layernorm output feeding the next GEMM
+  float* qkv;      // (M,3C)
+  float* atty;     // (M,C)
+  float* proj;     // (M,C) attproj / fcproj output
+  float* fch;      // (M,4C) gelu(fc)
+  float* logits;   // (M,V)
+  int last_B, last_T;
+};
+
+namespace g2 {
+
+static void free_activations(GPT2* m) {
+  void* ptrs[] = {m->ids, m->res_a, m->res_b, m->ln, m->qkv, m->atty, m->proj, m->fch, m->logits};
+  for (void* p : ptrs)
+    if (p) (void)hipFree(p);
+  m->ids = nullptr;
+  m->res_a = m->res_b = m->ln = m->qkv = m->atty = m->proj = m->fch = m->logits = nullptr;
+  m->cap_tokens = 0;
+}
+
+static int check_shape(const GPT2* m, int B, int T) {
+  if (!m) return fail(GPT2HIP_EINVAL, "gpt2: null model");
+  if (B < 1 || T < 1 || T > m->cfg.max_seq_len)
+    return fail(GPT2HIP_EINVAL, "gpt2: bad B=%d T=%d (max_seq_len %d)", B, T, m->cfg.max_seq_len);
+  if ((long long)B * T > (1LL << 24)) return fail(GPT2HIP_EINVAL, "gpt2: B*T=%lld too large", (long long)B * T);
+  return GPT2HIP_OK;
+}
+
+static int reserve(GPT2* m, int B, int T) {
+  if (int rc = check_shape(m, B, T)) return rc;
+  const long long M = (long long)B * T;
+  if (M <= m->cap_tokens) return GPT2HIP_OK;
+  free_activations(m);
+  const size_t C = m->cfg.channels, V = m->cfg.vocab_size, n = (size_t)M;
+  struct { void** p; size_t bytes; } want[] = {
+      {(void**)&m->ids, n * sizeof(int)},          {(void**)&m->res_a, n * C * 4},
+      {(void**)&m->res_b, n * C * 4},              {(void**)&m->ln, n * C * 4},
+      {(void**)&m->qkv, n * 3 * C * 4},            {(void**)&m->atty, n * C * 4},
+      {(void**)&m->proj, n * C * 4},               {(void**)&m->fch, n * 4 * C * 4},
+      {(void**)&m->logits, n * V * 4}};
+  for (auto& w : want) {
+    hipError_t e = hipMalloc(w.p, w.bytes);
+    if (e != hipSuccess) {
+      *w.p = nullptr;
+      free_activations(m);
+      return fail(GPT2HIP_ENOMEM, "gpt2: hipMalloc of %zu bytes failed: %s", w.bytes,
+                  hipGetErrorString(e));
+    }
+  }
+  m->cap_tokens = M;
+  return GPT2HIP_OK;
+}
+
+// The forward pass proper; ids are already in m->ids.
+static int forward_resident(GPT2* m, int B, int T) {
+  const GPT2Config& c = m->cfg;
+  const int C = c.channels, L = c.num_layers, NH = c.num_heads, V = c.vocab_size;
+  const size_t cs = (size_t)C;
+  auto P = [&](int which) { return m->params + m->param_off[which]; };
+#define G2_TRY(call)          \
+  do {                        \
+    if (int rc_ = (call)) return rc_; \
+  } while (0)
+
+  float* residual = m->res_a;  // current residual stream
+  float* other = m->res_b;
+  G2_TRY(encoder_forward_status(residual, m->ids, P(P_WTE), P(P_WPE), B, T, C));
+  // the one stand-alone layernorm: ln1 of layer 0
+  G2_TRY(layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, T, C));
+  for (int l = 0; l < L; l++) {
+    G2_TRY(matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
+                                 B, T, C, 3 * C));
+    G2_TRY(attention_forward_status(m->atty, nullptr, nullptr, m->qkv, B, T, C, NH));
+    G2_TRY(matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs,
+                                 P(P_ATTPROJB) + l * cs, B, T, C, C));
+    // residual2 = residual + attproj ; ln = ln2(residual2)
+    G2_TRY(fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual,
+                                                   m->proj, P(P_LN2W) + l * cs, P(P_LN2B) + l * cs,
+                                                   B, T, C));
+    G2_TRY(matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs,
+                                      P(P_FCB) + l * 4 * cs, B, T, C, 4 * C, 1));
+    G2_TRY(matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
+                                 P(P_FCPROJB) + l * cs, B, T, 4 * C, C));
+    // residual3 = residual2 + fcproj ; ln = ln1 of the next layer, or the final layernorm
+    const float* nw = (l + 1 < L) ? P(P_LN1W) + (l + 1) * cs : P(P_LNFW);
+    const float* nb = (l + 1 < L) ? P(P_LN1B) + (l + 1) * cs : P(P_LNFB);
+    G2_TRY(fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other,
+                                                   m->proj, nw, nb, B, T, C));
+  }
+  // lm-head: weight-tied to wte, no bias, unpadded vocabulary
+  G2_TRY(matmul_forward_status(m->logits, m->ln, P(P_WTE), nullptr, B, T, C, V));
+#undef G2_TRY
+  m->last_B = B;
+  m->last_T = T;
+  return GPT2HIP_OK;
+}
+
+}  // namespace g2
+
+extern "C" {
+
+const char* gpt2hip_last_error(void) { return g2::last_error_buffer(); }
+
+GPT2* gpt2_create(const GPT2Config* config) {
+  using namespace g2;
+  if (!config || config->max_seq_len < 1 || config->vocab_size < 1 || config->num_layers < 1 ||
+      config->num_heads < 1 || config->channels < 1 || config->channels % config->num_heads != 0) {
+    fail(GPT2HIP_EINVAL, "gpt2_create: invalid config");
+    return nullptr;
+  }
+  GPT2* m = new GPT2();
+  m->cfg = *config;
+  const size_t V = config->vocab_size, maxT = config->max_seq_len, L = config->num_layers,
+               C = config->channels;
+  const size_t sizes[P_COUNT] = {V * C,         maxT * C, L * C,         L * C,
+                                 L * 3 * C * C, L * 3 * C, L * C * C,     L * C,
+                                 L * C,         L * C,     L * 4 * C * C, L * 4 * C,
+                                 L * C * 4 * C, L * C,     C,             C};
+  size_t off = 0;
+  for (int i = 0; i < P_COUNT; i++) {
+    m->param_off[i] = off;
+    off += sizes[i];
+  }
+  m->num_params = off;
+  if (hipGetDevice(&m->device) != hipSuccess ||
+      hipMalloc((void**)&m->params, off * sizeof(float)) != hipSuccess) {
+    fail(GPT2HIP_ENOMEM, "gpt2_create: cannot allocate %zu parameter bytes", off * sizeof(float));
+    delete m;
+    return nullptr;
+  }
+  return m;
+}
+
+void gpt2_destroy(GPT2* model) {
+  if (!model) return;
+  g2::free_activations(model);
+  if (model->params) (void)hipFree(model->params);
+  delete model;
+}
+
+size_t gpt2_num_parameters(const GPT2* model) { return model ? model->num_params : 0; }
+float* gpt2_params_device(GPT2* model) { return model ? model->params : nullptr; }
+
+int gpt2_load_params_host(GPT2* model, const float* host_params, size_t n) {
+  using namespace g2;
+  if (!model || !host_params) return fail(GPT2HIP_EINVAL, "gpt2_load_params_host: null pointer");
+  if (n != model->num_params)
+    return fail(GPT2HIP_EINVAL, "gpt2_load_params_host: got %zu floats, model has %zu", n,
+                model->num_params);
+  G2_HIP(hipMemcpy(model->params, host_params, n * sizeof(float), hipMemcpyHostToDevice));
+  return GPT2HIP_OK;
+}
+
+int gpt2_reserve(GPT2* model, int B, int T) { return g2::reserve(model, B, T); }
+
+int gpt2_forward_status(GPT2* model, const int* inputs_host, int B, int T) {
+  using namespace g2;
+  if (int rc = reserve(model, B, T)) return rc;
+  if (!inputs_host) return fail(GPT2HIP_EINVAL, "gpt2_forward: null inputs");
+  const size_t n = (size_t)B * T;
+  for (size_t i = 0; i < n; i++)
+    if (inputs_host[i] < 0 || inputs_host[i] >= model->cfg.vocab_size)
+      return fail(GPT2HIP_EINVAL, "gpt2_forward: token id %d at position %zu outside [0,%d)",
+                  inputs_host[i], i, model->cfg.vocab_size);
+  G2_HIP(hipMemcpy(model->ids, inputs_host, n * sizeof(int), hipMemcpyHostToDevice));
+  return forward_resident(model, B, T);
+}
+
+void gpt2_forward(GPT2* model, const int* inputs_host, int B, int T) {
+  if (gpt2_forward_status(model, inputs_host, B, T)) g2::die("gpt2_forward");
+}
+
+int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int T) {
+  using namespace g2;
+  if (int rc = reserve(model, B, T)) return rc;
+  if (!inputs_device) return fail(GPT2HIP_EINVAL, "gpt2_forward_device: null inputs");
+  G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
+                        hipMemcpyDeviceToDevice, 0));
+  return forward_resident(model, B, T);
+}
+
+const float* gpt2_logits(const GPT2* model) { return model ? model->logits : nullptr; }
+const float* gpt2_lnf(const GPT2* model) { return model ? model->ln : nullptr; }
+
+int gpt2_argmax_status(GPT2* model, int* ids_device) {
+  using namespace g2;
+  if (!model || !model->logits || model->last_B == 0)
+    return fail(GPT2HIP_EINVAL, "gpt2_argmax: no forward pass has run");
+  return argmax_forward_status(ids_device, model->logits, model->last_B * model->last_T,
+                               model->cfg.vocab_size);
+}
+
+// ---- event timer on the null stream ---------------------------------------
+struct GPT2Timer {
+  hipEvent_t start, stop;
+};
+
+GPT2Timer* gpt2hip_timer_create(void) {
+  GPT2Timer* t = new GPT2Timer();
+  if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) {
+    g2::fail(GPT2HIP_EHIP, "gpt2hip_timer_create: hipEventCreate failed");
+    delete t;
+    return nullptr;
+  }
+  return t;
+}
+
+void gpt2hip_timer_destroy(GPT2Timer* t) {
+  if (!t) return;
+  (void)hipEventDestroy(t->start);
+  (void)hipEventDestroy(t->stop);
+  delete t;
+}
+
+int gpt2hip_timer_start(GPT2Timer* t) {
+  if (!t) return g2::fail(GPT2HIP_EINVAL, "gpt2hip_timer_start: null timer");
+  G2_HIP(hipEventRecord(t->start, 0));
+  return GPT2HIP_OK;
+}
+
+float gpt2hip_timer_stop_ms(GPT2Timer* t) {
+  if (!t) return -1.f;
+  float ms = -1.f;
+  if (hipEventRecord(t->stop, 0) != hipSuccess || hipEventSynchronize(t->stop) != hipSuccess ||
+      hipEventElapsedTime(&ms, t->start, t->stop) != hipSuccess) {
+    g2::fail(GPT2HIP_EHIP, "gpt2hip_timer_stop_ms: event timing failed");
+    return -1.f;
+  }
+  return ms;
+}
+
+}  // extern "C"

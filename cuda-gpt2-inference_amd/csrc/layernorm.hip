@@ -1,0 +1,191 @@
+// layernorm_forward and fused_residual_layernorm_forward for gfx950.
+//
+// One 64-lane wavefront owns one row.  The row (or the sum of the two input
+// rows) is read once with 128-bit loads and kept in registers; mean and
+// variance are two passes over those registers (llm.c's two-pass arithmetic,
+// not the E[x^2]-m^2 shortcut of reference 3_layernorm_warp.cuh:49-50), reduced
+// across the wave with DPP; the normalised row and, for the fused form, the
+// residual sum are written with 128-bit stores.  HBM traffic is the compulsory
+// one pass: 2 reads + 2 writes of the row for the fused form.
+#include "common.hpp"
+
+namespace g2 {
+
+constexpr int kRowsPerBlock = 4;  // 4 waves = 256 threads
+
+// NV float4 per lane cover C <= 256*NV.  FUSED adds inp2 and stores the sum.
+template <int NV, bool FUSED>
+__global__ __launch_bounds__(kRowsPerBlock* kWave) void layernorm_rows_kernel(
+    float* res_out, float* out, float* __restrict__ mean, float* __restrict__ rstd,
+    const float* inp1, const float* inp2, const float* __restrict__ weight,
+    const float* __restrict__ bias, int N, int C) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= N) return;
+  const int C4 = C >> 2;
+  const size_t base = (size_t)row * C4;
+  const f32x4* x1 = reinterpret_cast<const f32x4*>(inp1) + base;
+  const f32x4* x2 = FUSED ? reinterpret_cast<const f32x4*>(inp2) + base : nullptr;
+
+  f32x4 v[NV];
+#pragma unroll
+  for (int j = 0; j < NV; j++) {
+    const int c = lane + j * kWave;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+    if (c < C4) {
+      a = __builtin_nontemporal_load(x1 + c);
+      if (FUSED) a += __builtin_nontemporal_load(x2 + c);
+    }
+    v[j] = a;
+  }
+  if (FUSED) {
+    f32x4* ro = reinterpret_cast<f32x4*>(res_out) + base;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int c = lane + j * kWave;
+      if (c < C4) ro[c] = v[j];
+    }
+  }
+
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; j++) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+  const float m = wave_sum(s) / (float)C;
+
+  float q = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; j++) {
+    const int c = lane + j * kWave;
+    if (c < C4) {
+      const f32x4 d = v[j] - m;
+      q += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
+    }
+  }
+  const float var = wave_sum(q) / (float)C;
+  const float rs = 1.0f / sqrtf(var + 1e-5f);
+
+  if (lane == 0) {
+    if (mean) mean[row] = m;
+    if (rstd) rstd[row] = rs;
+  }
+
+  const f32x4* w4 = reinterpret_cast<const f32x4*>(weight);
+  const f32x4* b4 = reinterpret_cast<const f32x4*>(bias);
+  f32x4* o = reinterpret_cast<f32x4*>(out) + base;
+#pragma unroll
+  for (int j = 0; j < NV; j++) {
+    const int c = lane + j * kWave;
+    if (c < C4) {
+      const f32x4 n = (v[j] - m) * rs;
+      o[c] = n * w4[c] + b4[c];
+    }
+  }
+}
+
+// Any C, any alignment: one wave per row, three passes over global memory.
+template <bool FUSED>
+__global__ __launch_bounds__(kRowsPerBlock* kWave) void layernorm_rows_generic_kernel(
+    float* res_out, float* out, float* mean, float* rstd, const float* inp1, const float* inp2,
+    const float* weight, const float* bias, int N, int C) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= N) return;
+  const float* x1 = inp1 + (size_t)row * C;
+  const float* x2 = FUSED ? inp2 + (size_t)row * C : nullptr;
+  float* ro = FUSED ? res_out + (size_t)row * C : nullptr;
+  float s = 0.f;
+  for (int c = lane; c < C; c += kWave) {
+    float a = x1[c];
+    if (FUSED) {
+      a += x2[c];
+      ro[c] = a;  // each lane re-reads only what it wrote itself
+    }
+    s += a;
+  }
+  const float* x = FUSED ? ro : x1;
+  const float m = wave_sum(s) / (float)C;
+  float q = 0.f;
+  for (int c = lane; c < C; c += kWave) {
+    const float d = x[c] - m;
+    q += d * d;
+  }
+  const float rs = 1.0f / sqrtf(wave_sum(q) / (float)C + 1e-5f);
+  if (lane == 0) {
+    if (mean) mean[row] = m;
+    if (rstd) rstd[row] = rs;
+  }
+  float* o = out + (size_t)row * C;
+  for (int c = lane; c < C; c += kWave) o[c] = ((x[c] - m) * rs) * weight[c] + bias[c];
+}
+
+template <bool FUSED>
+static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd,
+                            const float* inp1, const float* inp2, const float* weight,
+                            const float* bias, int B, int T, int C) {
+  const char* name = FUSED ? "fused_residual_layernorm_forward" : "layernorm_forward";
+  if (B < 0 || T < 0 || C < 1) return fail(GPT2HIP_EINVAL, "%s: bad shape B=%d T=%d C=%d", name, B, T, C);
+  if (!out || !inp1 || !weight || !bias || (FUSED && (!res_out || !inp2)))
+    return fail(GPT2HIP_EINVAL, "%s: null pointer", name);
+  const long long N64 = (long long)B * T;
+  if (N64 > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "%s: B*T too large", name);
+  const int N = (int)N64;
+  if (N == 0) return GPT2HIP_OK;
+  const dim3 grid((N + kRowsPerBlock - 1) / kRowsPerBlock), block(kRowsPerBlock * kWave);
+  const bool vec = (C % 4 == 0) && C <= 4096 && aligned16(out) && aligned16(inp1) &&
+                   aligned16(weight) && aligned16(bias) &&
+                   (!FUSED || (aligned16(res_out) && aligned16(inp2)));
+#define G2_LN(NV)                                                                              \
+  hipLaunchKernelGGL((layernorm_rows_kernel<NV, FUSED>), grid, block, 0, 0, res_out, out, mean, \
+                     rstd, inp1, inp2, weight, bias, N, C)
+  if (!vec) {
+    hipLaunchKernelGGL((layernorm_rows_generic_kernel<FUSED>), grid, block, 0, 0, res_out, out,
+                       mean, rstd, inp1, inp2, weight, bias, N, C);
+  } else if (C <= 256) {
+    G2_LN(1);
+  } else if (C <= 512) {
+    G2_LN(2);
+  } else if (C <= 768) {
+    G2_LN(3);
+  } else if (C <= 1024) {
+    G2_LN(4);
+  } else if (C <= 2048) {
+    G2_LN(8);
+  } else {
+    G2_LN(16);
+  }
+#undef G2_LN
+  G2_LAUNCH_CHECK(name);
+  return GPT2HIP_OK;
+}
+
+}  // namespace g2
+
+extern "C" {
+
+int layernorm_forward_status(float* out, float* mean, float* rstd, const float* inp,
+                             const float* weight, const float* bias, int B, int T, int C) {
+  return g2::launch_layernorm<false>(nullptr, out, mean, rstd, inp, nullptr, weight, bias, B, T, C);
+}
+
+void layernorm_forward(float* out, float* mean, float* rstd, const float* inp, const float* weight,
+                       const float* bias, int B, int T, int C) {
+  if (layernorm_forward_status(out, mean, rstd, inp, weight, bias, B, T, C)) g2::die("layernorm_forward");
+}
+
+int fused_residual_layernorm_forward_status(float* res_out, float* layernorm_out, float* mean,
+                                            float* rstd, const float* inp1, const float* inp2,
+                                            const float* weight, const float* bias, int B, int T,
+                                            int C) {
+  return g2::launch_layernorm<true>(res_out, layernorm_out, mean, rstd, inp1, inp2, weight, bias, B,
+                                    T, C);
+}
+
+void fused_residual_layernorm_forward(float* res_out, float* layernorm_out, float* mean,
+                                      float* rstd, const float* inp1, const float* inp2,
+                                      const float* weight, const float* bias, int B, int T, int C) {
+  if (fused_residual_layernorm_forward_status(res_out, layernorm_out, mean, rstd, inp1, inp2,
+                                              weight, bias, B, T, C))
+    g2::die("fused_residual_layernorm_forward");
+}
+
+}  // extern "C"

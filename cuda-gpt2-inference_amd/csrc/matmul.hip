@@ -1,0 +1,292 @@
+// matmul_forward for gfx950: out(M,N) = inp(M,K) . weight(N,K)^T + bias(N),
+// optional tanh-GELU epilogue.  True fp32 on the matrix cores
+// (v_mfma_f32_32x32x2_f32; gfx950 has no xf32 path).
+//
+// Tiling.  A workgroup owns a BM x BN output tile and walks K in slabs of
+// BK = 32.  Both operands are K-contiguous in memory ("NT" GEMM), so a slab of
+// either is rows of 32 floats = 8 chunks of 16 bytes.  Slabs are fetched with
+// 128-bit global loads into registers one slab ahead, then stored to one of
+// two LDS buffers; one barrier per slab.  In LDS, chunk c of row r sits at
+// chunk position c ^ (r & 7): eight lanes that read the same logical chunk of
+// eight consecutive rows then hit eight different 16-byte bank groups, which
+// makes both the 128-bit stores and the 128-bit operand reads conflict-free.
+//
+// MFMA operand mapping.  v_mfma_f32_32x32x2_f32 takes A[i][k] from lane
+// (i = lane%32, k = lane/32) and B[k][j] from lane (j = lane%32, k = lane/32).
+// A lane with h = lane/32 reads the 16-byte chunk 2g+h of its row, i.e.
+// k = 8g+4h .. 8g+4h+3, and feeds element s of it to the s-th of four MFMAs:
+// that MFMA multiplies k = 8g+s (lanes 0..31) and k = 8g+4+s (lanes 32..63).
+// A and B use the same k permutation, so the contraction is unchanged and one
+// ds_read_b128 per 32 rows feeds four MFMAs.
+//
+// The accumulator of lane l, register v holds D[8*(v/4) + 4*(l/32) + v%4][l%32]:
+// a lane owns one output column, so the bias is folded into the accumulator's
+// initial value (as the reference does, 9_matmul_async_cg_tf32_gelu.cuh:56-84)
+// and every store instruction writes two 128-byte row segments.
+#include "common.hpp"
+
+namespace g2 {
+
+constexpr int BK = 32;           // floats per K slab
+constexpr int CHUNKS = BK / 4;   // 16-byte chunks per slab row
+
+// Workgroup -> tile.  Hardware deals consecutive workgroup ids round-robin to
+// the 8 XCDs (each with a private L2).  When the number of row tiles divides by
+// 8, XCD x is given the band of row tiles [x*band, (x+1)*band) and walks it
+// column tile by column tile, so that the band's A rows stay in that XCD's L2
+// and each B column tile is fetched once per XCD.
+__device__ __forceinline__ void tile_of_block(int pid, int ntm, int ntn, int& tm, int& tn) {
+  if ((ntm & 7) == 0) {
+    const int band = ntm >> 3;
+    const int xcd = pid & 7;
+    const int q = pid >> 3;
+    tm = xcd * band + q % band;
+    tn = q / band;
+  } else {
+    tm = pid % ntm;
+    tn = pid / ntm;
+  }
+}
+
+template <int BM, int BN, int WGM, int WGN, bool GELU>
+__global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
+    float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
+    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn) {
+  constexpr int NT = WGM * WGN * kWave;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_PER = BM * CHUNKS / NT, B_PER = BN * CHUNKS / NT;
+  static_assert(BM * CHUNKS % NT == 0 && BN * CHUNKS % NT == 0, "tile/threads mismatch");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be 32x32 MFMA tiles");
+  constexpr int STAGE = (BM + BN) * CHUNKS;  // f32x4 per LDS buffer
+
+  extern __shared__ f32x4 lds[];  // [2][STAGE]: A rows then B rows
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, ntm, ntn, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // ---- global -> register staging --------------------------------------
+  // chunk q = tid + j*NT of the slab: row q/8, chunk q%8.
+  const float* a_src[A_PER];
+  const float* b_src[B_PER];
+  int a_dst[A_PER], b_dst[B_PER];
+  const int kc = (tid & 7) * 4;  // this thread's k offset inside a slab (same for all j)
+#pragma unroll
+  for (int j = 0; j < A_PER; j++) {
+    const int q = tid + j * NT;
+    const int r = q >> 3, c = q & 7;
+    const int gm = m0 + r;
+    a_src[j] = (gm < M) ? inp + (size_t)gm * K + kc : nullptr;
+    a_dst[j] = r * CHUNKS + (c ^ (r & 7));
+  }
+#pragma unroll
+  for (int j = 0; j < B_PER; j++) {
+    const int q = tid + j * NT;
+    const int r = q >> 3, c = q & 7;
+    const int gn = n0 + r;
+    b_src[j] = (gn < N) ? weight + (size_t)gn * K + kc : nullptr;
+    b_dst[j] = BM * CHUNKS + r * CHUNKS + (c ^ (r & 7));
+  }
+
+  f32x4 a_reg[A_PER], b_reg[B_PER];
+  auto fetch = [&](int k0) {
+    const bool kin = (k0 + kc) < K;  // K is a multiple of 4: a chunk is all in or all out
+#pragma unroll
+    for (int j = 0; j < A_PER; j++) {
+      f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      if (kin && a_src[j]) z = *reinterpret_cast<const f32x4*>(a_src[j] + k0);
+      a_reg[j] = z;
+    }
+#pragma unroll
+    for (int j = 0; j < B_PER; j++) {
+      f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      if (kin && b_src[j]) z = *reinterpret_cast<const f32x4*>(b_src[j] + k0);
+      b_reg[j] = z;
+    }
+  };
+  auto stash = [&](int buf) {
+    f32x4* s = lds + buf * STAGE;
+#pragma unroll
+    for (int j = 0; j < A_PER; j++) s[a_dst[j]] = a_reg[j];
+#pragma unroll
+    for (int j = 0; j < B_PER; j++) s[b_dst[j]] = b_reg[j];
+  };
+
+  // ---- accumulators, initialised with the bias of the lane's column ----
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int col = n0 + wn * WN + j * 32 + (lane & 31);
+    const float bv = (bias != nullptr && col < N) ? bias[col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = bv;
+  }
+
+  // ---- operand read offsets (f32x4 units) inside an LDS buffer ----------
+  // row & 7 == lane & 7 because every row base is a multiple of 32.
+  const int h = lane >> 5;
+  const int sw = lane & 7;
+  int a_row[TM], b_row[TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++) a_row[i] = (wm * WM + i * 32 + (lane & 31)) * CHUNKS;
+#pragma unroll
+  for (int j = 0; j < TN; j++) b_row[j] = BM * CHUNKS + (wn * WN + j * 32 + (lane & 31)) * CHUNKS;
+
+  const int nslab = (K + BK - 1) / BK;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+
+  for (int s = 0; s < nslab; s++) {
+    const f32x4* cur = lds + (s & 1) * STAGE;
+    if (s + 1 < nslab) fetch((s + 1) * BK);
+
+    f32x4 af[2][TM], bf[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) af[0][i] = cur[a_row[i] + ((0 + h) ^ sw)];
+#pragma unroll
+    for (int j = 0; j < TN; j++) bf[0][j] = cur[b_row[j] + ((0 + h) ^ sw)];
+#pragma unroll
+    for (int g = 0; g < CHUNKS / 2; g++) {
+      const int p = g & 1;
+      if (g + 1 < CHUNKS / 2) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) af[p ^ 1][i] = cur[a_row[i] + ((2 * (g + 1) + h) ^ sw)];
+#pragma unroll
+        for (int j = 0; j < TN; j++) bf[p ^ 1][j] = cur[b_row[j] + ((2 * (g + 1) + h) ^ sw)];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[p][i][e], bf[p][j][e], acc[i][j], 0,
+                                                             0, 0);
+    }
+
+    if (s + 1 < nslab) stash((s + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue -----------------------------------------------------------
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int col = n0 + wn * WN + j * 32 + (lane & 31);
+      const int rbase = m0 + wm * WM + i * 32 + 4 * h;
+      if (col < N) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int row = rbase + 8 * (v >> 2) + (v & 3);
+          if (row < M) {
+            float r = acc[i][j][v];
+            if (GELU) r = gelu_tanh(r);
+            out[(size_t)row * N + col] = r;
+          }
+        }
+      }
+    }
+  }
+}
+
+// Any shape, any alignment; one thread per output.  Only used when K is not a
+// multiple of 4 or an operand is not 16-byte aligned.
+__global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const float* inp,
+                                                              const float* weight,
+                                                              const float* bias, int M, int K, int N,
+                                                              int gelu) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)M * N) return;
+  const int row = (int)(idx / N), col = (int)(idx % N);
+  const float* x = inp + (size_t)row * K;
+  const float* w = weight + (size_t)col * K;
+  float acc = bias ? bias[col] : 0.f;
+  for (int k = 0; k < K; k++) acc += x[k] * w[k];
+  out[idx] = gelu ? gelu_tanh(acc) : acc;
+}
+
+template <int BM, int BN, int WGM, int WGN>
+static int launch_mfma(float* out, const float* inp, const float* weight, const float* bias, int M,
+                       int K, int N, bool gelu) {
+  constexpr int NT = WGM * WGN * kWave;
+  constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
+  const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
+  const long long tiles = (long long)ntm * ntn;
+  if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
+  auto kfn = gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true>
+                  : matmul_mfma_kernel<BM, BN, WGM, WGN, false>;
+  static thread_local int configured_for = -1;  // device whose attribute was set (per variant)
+  static thread_local int configured_mask = 0;
+  int dev = 0;
+  G2_HIP(hipGetDevice(&dev));
+  if (configured_for != dev) {
+    configured_for = dev;
+    configured_mask = 0;
+  }
+  const int bit = gelu ? 2 : 1;
+  if (!(configured_mask & bit)) {
+    G2_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    configured_mask |= bit;
+  }
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
+                     K, N, ntm, ntn);
+  G2_LAUNCH_CHECK("matmul_forward");
+  return GPT2HIP_OK;
+}
+
+static int matmul_dispatch(float* out, const float* inp, const float* weight, const float* bias,
+                           int B, int T, int C, int OC, bool gelu) {
+  if (B < 0 || T < 0 || C < 1 || OC < 1)
+    return fail(GPT2HIP_EINVAL, "matmul_forward: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
+  if (!out || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward: null pointer");
+  const long long M64 = (long long)B * T;
+  if (M64 > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: B*T too large");
+  const int M = (int)M64;
+  if (M == 0) return GPT2HIP_OK;
+  if (C % 4 != 0 || !aligned16(inp) || !aligned16(weight)) {
+    const size_t total = (size_t)M * OC;
+    hipLaunchKernelGGL(matmul_generic_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, 0,
+                       out, inp, weight, bias, M, C, OC, gelu ? 1 : 0);
+    G2_LAUNCH_CHECK("matmul_forward");
+    return GPT2HIP_OK;
+  }
+  return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu);
+}
+
+}  // namespace g2
+
+extern "C" {
+
+int matmul_forward_status(float* out, const float* inp, const float* weight, const float* bias,
+                          int B, int T, int C, int OC) {
+  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false);
+}
+
+void matmul_forward(float* out, const float* inp, const float* weight, const float* bias, int B,
+                    int T, int C, int OC) {
+  if (matmul_forward_status(out, inp, weight, bias, B, T, C, OC)) g2::die("matmul_forward");
+}
+
+int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,
+                               const float* bias, int B, int T, int C, int OC, int is_gelu) {
+  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, is_gelu != 0);
+}
+
+void matmul_forward_gelu(float* out, const float* inp, const float* weight, const float* bias,
+                         int B, int T, int C, int OC, int is_gelu) {
+  if (matmul_forward_gelu_status(out, inp, weight, bias, B, T, C, OC, is_gelu))
+    g2::die("matmul_forward_gelu");
+}
+
+}  // extern "C"

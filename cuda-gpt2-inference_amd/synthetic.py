@@ -1,0 +1,60 @@
+"""Seeded synthetic GPT-2 parameters and token ids (host side, numpy).
+
+There are no checkpoints offline, so weights follow GPT-2's initialisation:
+N(0, 0.02) for wte / qkvw / fcw, the two residual projections scaled by
+1/sqrt(2L), wpe N(0, 0.01), layernorm gamma 1 / beta 0, biases 0.  The flat
+buffer is in llm.c checkpoint order (the order gpt2_params_device() documents).
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+PARAM_NAMES = ("wte", "wpe", "ln1w", "ln1b", "qkvw", "qkvb", "attprojw", "attprojb", "ln2w",
+               "ln2b", "fcw", "fcb", "fcprojw", "fcprojb", "lnfw", "lnfb")
+
+
+def param_shapes(*, max_seq_len, vocab_size, num_layers, num_heads, channels):
+    V, maxT, L, C = vocab_size, max_seq_len, num_layers, channels
+    return {
+        "wte": (V, C), "wpe": (maxT, C), "ln1w": (L, C), "ln1b": (L, C),
+        "qkvw": (L, 3 * C, C), "qkvb": (L, 3 * C), "attprojw": (L, C, C), "attprojb": (L, C),
+        "ln2w": (L, C), "ln2b": (L, C), "fcw": (L, 4 * C, C), "fcb": (L, 4 * C),
+        "fcprojw": (L, C, 4 * C), "fcprojb": (L, C), "lnfw": (C,), "lnfb": (C,),
+    }
+
+
+def make_params(seed: int, *, perturb_affine: bool = False, **config) -> np.ndarray:
+    """Flat float32 parameter buffer.  perturb_affine also randomises the
+    layernorm affine terms and the biases (so tests exercise them)."""
+    shapes = param_shapes(**config)
+    L = config["num_layers"]
+    rng = np.random.default_rng(seed)
+    total = sum(int(np.prod(s)) for s in shapes.values())
+    flat = np.empty(total, np.float32)
+    off = 0
+    for name in PARAM_NAMES:
+        n = int(np.prod(shapes[name]))
+        dst = flat[off:off + n]
+        if name in ("wte", "qkvw", "fcw"):
+            dst[:] = rng.standard_normal(n, dtype=np.float32) * np.float32(0.02)
+        elif name in ("attprojw", "fcprojw"):
+            dst[:] = rng.standard_normal(n, dtype=np.float32) * np.float32(0.02 / math.sqrt(2 * L))
+        elif name == "wpe":
+            dst[:] = rng.standard_normal(n, dtype=np.float32) * np.float32(0.01)
+        elif name in ("ln1w", "ln2w", "lnfw"):
+            dst[:] = 1.0
+            if perturb_affine:
+                dst += rng.standard_normal(n, dtype=np.float32) * np.float32(0.1)
+        else:  # layernorm betas and linear biases
+            dst[:] = 0.0
+            if perturb_affine:
+                dst += rng.standard_normal(n, dtype=np.float32) * np.float32(0.02)
+        off += n
+    return flat
+
+
+def make_tokens(seed: int, B: int, T: int, vocab_size: int) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return rng.integers(0, vocab_size, (B, T), dtype=np.int32)

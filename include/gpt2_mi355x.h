@@ -1,0 +1,163 @@
+/*
+ * C ABI of the MI355X (gfx950) GPT-2 fp32 forward library, libgpt2_mi355x.so.
+ *
+ * The entry points keep the llm.c launcher convention that the reference's
+ * kernels are drop-ins for: raw device pointers + int dims, caller owns every
+ * buffer, launches go to the null stream in order, nothing synchronises and
+ * nothing is allocated inside a launcher.  Each launcher exists in two forms:
+ *
+ *   int  <name>_status(...)   returns 0 or a GPT2HIP_E* code (message via
+ *                             gpt2hip_last_error()); never aborts.
+ *   void <name>(...)          the llm.c form: prints the message and aborts on
+ *                             failure, like llm.c's cudaCheck / the reference's
+ *                             assert()s.
+ *
+ * All tensors are fp32, row-major, device memory.  Rows do not need padding.
+ */
+#ifndef GPT2_MI355X_H
+#define GPT2_MI355X_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  GPT2HIP_OK = 0,
+  GPT2HIP_EINVAL = 1, /* bad shape or null pointer */
+  GPT2HIP_EHIP = 2,   /* a HIP runtime call failed */
+  GPT2HIP_ENOMEM = 3
+};
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* gpt2hip_last_error(void);
+
+/* out[b,t,:] = wte[inp[b,t],:] + wpe[t,:].  inp is int32 (B,T) on the device.
+ * Replaces llm.c's encoder_forward, which the reference leaves untouched
+ * (named in reference README.md:10). */
+int encoder_forward_status(float* out, const int* inp, const float* wte, const float* wpe, int B,
+                           int T, int C);
+void encoder_forward(float* out, const int* inp, const float* wte, const float* wpe, int B, int T,
+                     int C);
+
+/* Row-wise layernorm, eps 1e-5; mean/rstd (B*T) may be NULL.
+ * Replaces layernorm_forward_warp, reference
+ * kernels/layernorm/3_layernorm_warp.cuh:78-80. */
+int layernorm_forward_status(float* out, float* mean, float* rstd, const float* inp,
+                             const float* weight, const float* bias, int B, int T, int C);
+void layernorm_forward(float* out, float* mean, float* rstd, const float* inp, const float* weight,
+                       const float* bias, int B, int T, int C);
+
+/* res_out = inp1 + inp2; layernorm_out = layernorm(res_out); mean/rstd may be
+ * NULL.  res_out may alias inp1 or inp2.  Replaces
+ * fused_residual_layernorm_forward, reference
+ * kernels/fused_residual_layernorm/fused_residual_layernorm.cuh:88-90. */
+int fused_residual_layernorm_forward_status(float* res_out, float* layernorm_out, float* mean,
+                                            float* rstd, const float* inp1, const float* inp2,
+                                            const float* weight, const float* bias, int B, int T,
+                                            int C);
+void fused_residual_layernorm_forward(float* res_out, float* layernorm_out, float* mean,
+                                      float* rstd, const float* inp1, const float* inp2,
+                                      const float* weight, const float* bias, int B, int T, int C);
+
+/* out = inp1 + inp2 over N floats.  Replaces residual_forward_naive, reference
+ * kernels/residual/1_residual_naive.cuh:15. */
+int residual_forward_status(float* out, const float* inp1, const float* inp2, int N);
+void residual_forward(float* out, const float* inp1, const float* inp2, int N);
+
+/* tanh-GELU over N floats (llm.c's gelu_forward; the reference only has the
+ * device function, kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:5-11).
+ * size_t form for N above INT_MAX is not needed at GPT-2 sizes. */
+int gelu_forward_status(float* out, const float* inp, int N);
+void gelu_forward(float* out, const float* inp, int N);
+
+/* out(B*T,OC) = inp(B*T,C) . weight(OC,C)^T + bias(OC); bias may be NULL.
+ * Any B*T, C, OC >= 1.  Replaces matmul_forward_cublas, reference
+ * kernels/matmul/2_matmul_cublas.cuh:34-42 (and the other numbered attempts,
+ * which share the signature). */
+int matmul_forward_status(float* out, const float* inp, const float* weight, const float* bias,
+                          int B, int T, int C, int OC);
+void matmul_forward(float* out, const float* inp, const float* weight, const float* bias, int B,
+                    int T, int C, int OC);
+
+/* Same with tanh-GELU applied to the result when is_gelu != 0.  Replaces
+ * matmul_forward_async_cg_tf32_gelu, reference
+ * kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:237-246. */
+int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,
+                               const float* bias, int B, int T, int C, int OC, int is_gelu);
+void matmul_forward_gelu(float* out, const float* inp, const float* weight, const float* bias,
+                         int B, int T, int C, int OC, int is_gelu);
+
+/* Causal multi-head self-attention.  inp is packed qkv (B,T,3C): q at column
+ * 0, k at +C, v at +2C, head h at h*(C/NH) inside each; out is (B,T,C).
+ * qkvr and att are the llm.c scratch arguments: ignored, may be NULL.  inp is
+ * never written.  Replaces flash_attention_permute_forward, reference
+ * kernels/attention/3_flash_attention_permute.cuh:346-351. */
+int attention_forward_status(float* out, float* qkvr, float* att, const float* inp, int B, int T,
+                             int C, int NH);
+void attention_forward(float* out, float* qkvr, float* att, const float* inp, int B, int T, int C,
+                       int NH);
+
+/* ids[r] = argmax_v logits[r,v] for N rows of V floats; lowest index wins ties.
+ * No counterpart in the reference (llm.c samples on the host); needed for the
+ * "argmax ids" output of the forward pass. */
+int argmax_forward_status(int* ids, const float* logits, int N, int V);
+void argmax_forward(int* ids, const float* logits, int N, int V);
+
+/* ---- whole model: the gpt2_forward driver (llm.c train_gpt2_fp32.cu's
+ * gpt2_forward, which the reference plugs its kernels into, README.md:19;
+ * dataflow in reference images/gpt2/gpt2_flow.png). ---- */
+
+typedef struct {
+  int max_seq_len; /* maxT */
+  int vocab_size;  /* V    */
+  int num_layers;  /* L    */
+  int num_heads;   /* NH   */
+  int channels;    /* C    */
+} GPT2Config;
+
+typedef struct GPT2 GPT2; /* opaque */
+
+/* Allocates the parameter buffer (uninitialised) on the current device.
+ * Returns NULL on failure (see gpt2hip_last_error). */
+GPT2* gpt2_create(const GPT2Config* config);
+void gpt2_destroy(GPT2* model);
+
+/* Number of fp32 parameters, and the flat device buffer that holds them in
+ * llm.c checkpoint order: wte(V,C) wpe(maxT,C) ln1w(L,C) ln1b(L,C)
+ * qkvw(L,3C,C) qkvb(L,3C) attprojw(L,C,C) attprojb(L,C) ln2w(L,C) ln2b(L,C)
+ * fcw(L,4C,C) fcb(L,4C) fcprojw(L,C,4C) fcprojb(L,C) lnfw(C) lnfb(C). */
+size_t gpt2_num_parameters(const GPT2* model);
+float* gpt2_params_device(GPT2* model);
+/* Copies n = gpt2_num_parameters floats from host memory into that buffer. */
+int gpt2_load_params_host(GPT2* model, const float* host_params, size_t n);
+
+/* Allocates activations for up to B*T tokens (forward does this on demand; call
+ * it up front to keep allocation out of a timed region). */
+int gpt2_reserve(GPT2* model, int B, int T);
+
+/* Forward pass.  gpt2_forward takes HOST token ids like llm.c and copies them
+ * in; gpt2_forward_device takes ids already on the device.  Afterwards
+ * gpt2_logits() is (B,T,V) on the device.  Launches are asynchronous. */
+int gpt2_forward_status(GPT2* model, const int* inputs_host, int B, int T);
+void gpt2_forward(GPT2* model, const int* inputs_host, int B, int T);
+int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int T);
+const float* gpt2_logits(const GPT2* model);
+/* Final layernorm output (B,T,C) of the last forward, on the device. */
+const float* gpt2_lnf(const GPT2* model);
+/* Per-position argmax of the last forward's logits into ids_device (B*T). */
+int gpt2_argmax_status(GPT2* model, int* ids_device);
+
+/* Event timer on the null stream (the stream every launcher uses). */
+typedef struct GPT2Timer GPT2Timer;
+GPT2Timer* gpt2hip_timer_create(void);
+void gpt2hip_timer_destroy(GPT2Timer* t);
+int gpt2hip_timer_start(GPT2Timer* t);
+/* Records the stop event, waits for it, returns elapsed ms (negative on error). */
+float gpt2hip_timer_stop_ms(GPT2Timer* t);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPT2_MI355X_H */

@@ -1,0 +1,71 @@
+"""CPU-only checks of the drop-in boundary: the shared library loads, exports
+every symbol the public header declares, and the Python mirror refuses to run
+without device memory (no silent fallback)."""
+import ctypes
+import importlib
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+g2 = importlib.import_module("cuda-gpt2-inference_amd")
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "gpt2_mi355x.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b([a-z][a-z0-9_]*)\s*\(", text)
+    return sorted({n for n in names if n not in ("defined",)})
+
+
+def test_header_and_python_export_lists_agree():
+    assert declared_symbols() == sorted(g2.EXPORTS)
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(g2.LIB_PATH), "build with __graft_entry__.build() first"
+    L = ctypes.CDLL(g2.LIB_PATH)
+    missing = [s for s in declared_symbols() if not hasattr(L, s)]
+    assert not missing, missing
+
+
+def test_last_error_is_a_string():
+    assert isinstance(g2.lib().gpt2hip_last_error(), bytes)
+
+
+def test_launchers_reject_host_memory():
+    a = np.zeros(8, np.float32)
+    with pytest.raises(TypeError):
+        g2.residual_forward(a, a, a, 8)
+
+
+def test_shape_errors_are_reported_not_aborted():
+    # Argument validation happens before any HIP call, so it runs without a GPU.
+    L = g2.lib()
+    fake = ctypes.c_void_p(4096)
+    assert L.matmul_forward_status(fake, fake, fake, None, 1, 1, 0, 8) == 1
+    assert b"bad shape" in L.gpt2hip_last_error()
+    assert L.matmul_forward_status(None, fake, fake, None, 1, 1, 8, 8) == 1
+    assert L.attention_forward_status(fake, None, None, fake, 1, 8, 30, 4) == 1  # C % NH != 0
+    assert L.layernorm_forward_status(fake, None, None, fake, fake, None, 1, 1, 8) == 1
+    assert L.residual_forward_status(fake, fake, None, 8) == 1
+    assert L.argmax_forward_status(fake, fake, 1, 0) == 1
+    assert L.encoder_forward_status(fake, fake, fake, fake, 1, 1, 0) == 1
+    # empty work is a no-op, not an error
+    assert L.residual_forward_status(fake, fake, fake, 0) == 0
+    assert L.matmul_forward_status(fake, fake, fake, None, 0, 5, 8, 8) == 0
+
+
+def test_synthetic_params_match_oracle_layout():
+    import oracle
+    syn = importlib.import_module("cuda-gpt2-inference_amd.synthetic")
+    cfg = dict(max_seq_len=16, vocab_size=97, num_layers=2, num_heads=2, channels=32)
+    p = syn.make_params(0, **cfg)
+    assert p.size == oracle.num_parameters(16, 97, 2, 32)
+    sizes = oracle.param_sizes(16, 97, 2, 32)
+    shapes = syn.param_shapes(**cfg)
+    assert list(sizes) == list(syn.PARAM_NAMES)
+    for k in sizes:
+        assert sizes[k] == int(np.prod(shapes[k]))

@@ -1,0 +1,345 @@
+"""GPU parity: every launcher, called through the C ABI, against the CPU oracle
+on the same seeded inputs.
+
+Bar: bit-exact for the embedding gather, the residual add and argmax;
+|gpu - cpu| <= 1e-5 + 1e-4*|cpu| for every floating-point kernel.
+"""
+import importlib
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+g2 = importlib.import_module("cuda-gpt2-inference_amd")
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_close(gpu, cpu, what):
+    gpu = gpu.detach().cpu().numpy() if isinstance(gpu, torch.Tensor) else gpu
+    assert gpu.shape == cpu.shape, (what, gpu.shape, cpu.shape)
+    err = np.abs(gpu.astype(np.float64) - cpu.astype(np.float64))
+    tol = ATOL + RTOL * np.abs(cpu.astype(np.float64))
+    bad = err > tol
+    if bad.any() or not np.isfinite(gpu).all():
+        i = np.unravel_index(np.argmax(err - tol), err.shape)
+        raise AssertionError(f"{what}: {bad.sum()} of {bad.size} outside tolerance; worst at {i}: "
+                             f"gpu={gpu[i]!r} cpu={cpu[i]!r} err={err[i]:.3e} tol={tol[i]:.3e}")
+    return float(err.max())
+
+
+def guard(shape, dtype=torch.float32):
+    """Output buffer with NaN guard bands on both sides to catch stray writes."""
+    n = int(np.prod(shape))
+    pad = 1024
+    full = torch.full((n + 2 * pad,), float("nan") if dtype == torch.float32 else -7,
+                      dtype=dtype, device="cuda")
+    return full, full[pad:pad + n].view(*shape), pad
+
+
+def check_guard(full, pad):
+    head, tail = full[:pad], full[-pad:]
+    if full.dtype == torch.float32:
+        assert torch.isnan(head).all() and torch.isnan(tail).all(), "write outside the output"
+    else:
+        assert (head == -7).all() and (tail == -7).all(), "write outside the output"
+
+
+# ------------------------------------------------------------------ encoder
+@pytest.mark.parametrize("B,T,C,V", [(4, 64, 768, 50257), (2, 5, 12, 11), (3, 7, 10, 13),
+                                     (8, 1024, 768, 50257)])
+def test_encoder_bit_exact(B, T, C, V):
+    say(f"encoder B={B} T={T} C={C} V={V}")
+    r = np.random.default_rng(100)
+    wte = r.standard_normal((V, C), dtype=np.float32) * np.float32(0.02)
+    wpe = r.standard_normal((max(T, 8), C), dtype=np.float32) * np.float32(0.01)
+    ids = r.integers(0, V, (B, T), dtype=np.int32)
+    full, out, pad = guard((B, T, C))
+    g2.encoder_forward(out, dev(ids), dev(wte), dev(wpe), B, T, C)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    assert np.array_equal(out.cpu().numpy(), oracle.encoder_forward(ids, wte, wpe))
+
+
+# ------------------------------------------------------------------ residual / gelu
+@pytest.mark.parametrize("N", [0, 1, 3, 4, 1023, 4096 + 5, 8192 * 768])
+def test_residual_bit_exact(N):
+    say(f"residual N={N}")
+    r = np.random.default_rng(101)
+    a = r.standard_normal(N, dtype=np.float32)
+    b = r.standard_normal(N, dtype=np.float32)
+    full, out, pad = guard((N,))
+    g2.residual_forward(out, dev(a), dev(b), N)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    assert np.array_equal(out.cpu().numpy(), oracle.residual_forward(a, b))
+
+
+def test_residual_unaligned_pointers():
+    N = 1001
+    r = np.random.default_rng(102)
+    a = r.standard_normal(N + 1, dtype=np.float32)
+    b = r.standard_normal(N + 1, dtype=np.float32)
+    da, db = dev(a), dev(b)
+    out = torch.zeros(N + 1, device="cuda")
+    g2.residual_forward(out[1:], da[1:], db[1:], N)  # 4-byte aligned only
+    assert np.array_equal(out[1:].cpu().numpy(), a[1:] + b[1:])
+    assert out[0].item() == 0.0
+
+
+@pytest.mark.parametrize("N", [1, 7, 4096 + 3, 8192 * 3072])
+def test_gelu(N):
+    say(f"gelu N={N}")
+    r = np.random.default_rng(103)
+    x = r.standard_normal(N, dtype=np.float32) * np.float32(3.0)
+    full, out, pad = guard((N,))
+    g2.gelu_forward(out, dev(x), N)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    assert_close(out, oracle.gelu_forward(x), "gelu")
+
+
+def test_gelu_special_values():
+    x = np.array([0.0, -0.0, 30.0, -30.0, 1e-20, 88.0, -88.0], np.float32)
+    out = torch.empty(x.size, device="cuda")
+    g2.gelu_forward(out, dev(x), x.size)
+    assert_close(out, oracle.gelu_forward(x), "gelu special")
+
+
+# ------------------------------------------------------------------ layernorm
+def ln_inputs(N, C, seed):
+    r = np.random.default_rng(seed)
+    x = r.standard_normal((N, C), dtype=np.float32)
+    res = r.standard_normal((N, C), dtype=np.float32)
+    w = (1 + 0.1 * r.standard_normal(C)).astype(np.float32)
+    b = (0.1 * r.standard_normal(C)).astype(np.float32)
+    return x, res, w, b
+
+
+@pytest.mark.parametrize("N,C", [(8192, 768), (8192, 1024), (256, 768), (5, 64), (7, 260),
+                                 (3, 2048), (2, 4096), (9, 4100), (6, 50), (1, 1)])
+def test_layernorm(N, C):
+    say(f"layernorm N={N} C={C}")
+    x, _, w, b = ln_inputs(N, C, 110)
+    fo, out, po = guard((N, C))
+    fm, mean, pm = guard((N,))
+    fr, rstd, pr = guard((N,))
+    g2.layernorm_forward(out, mean, rstd, dev(x), dev(w), dev(b), 1, N, C)
+    torch.cuda.synchronize()
+    for f, p in ((fo, po), (fm, pm), (fr, pr)):
+        check_guard(f, p)
+    eo, em, er = oracle.layernorm_forward(x, w, b)
+    assert_close(out, eo, "layernorm out")
+    assert_close(mean, em, "layernorm mean")
+    assert_close(rstd, er, "layernorm rstd")
+
+
+def test_layernorm_null_stats_and_constant_row():
+    N, C = 4, 768
+    x = np.full((N, C), 3.25, np.float32)
+    _, _, w, b = ln_inputs(N, C, 111)
+    out = torch.empty((N, C), device="cuda")
+    g2.layernorm_forward(out, None, None, dev(x), dev(w), dev(b), 2, 2, C)
+    assert np.array_equal(out.cpu().numpy(), np.broadcast_to(b, (N, C)))
+
+
+@pytest.mark.parametrize("N,C", [(8192, 768), (8192, 1024), (256, 768), (5, 64), (7, 260),
+                                 (3, 2048), (9, 4100), (6, 50)])
+def test_fused_residual_layernorm(N, C):
+    say(f"fused_residual_layernorm N={N} C={C}")
+    x, res, w, b = ln_inputs(N, C, 112)
+    fo, out, po = guard((N, C))
+    fs, rsum, ps = guard((N, C))
+    fm, mean, pm = guard((N,))
+    fr, rstd, pr = guard((N,))
+    g2.fused_residual_layernorm_forward(rsum, out, mean, rstd, dev(x), dev(res), dev(w), dev(b), 1,
+                                        N, C)
+    torch.cuda.synchronize()
+    for f, p in ((fo, po), (fs, ps), (fm, pm), (fr, pr)):
+        check_guard(f, p)
+    es, eo, em, er = oracle.fused_residual_layernorm_forward(x, res, w, b)
+    assert np.array_equal(rsum.cpu().numpy(), es), "residual sum must be bit-exact"
+    assert_close(out, eo, "fused ln out")
+    assert_close(mean, em, "fused mean")
+    assert_close(rstd, er, "fused rstd")
+
+
+def test_fused_residual_layernorm_in_place_residual():
+    N, C = 300, 768
+    x, res, w, b = ln_inputs(N, C, 113)
+    dx = dev(x)
+    out = torch.empty((N, C), device="cuda")
+    g2.fused_residual_layernorm_forward(dx, out, None, None, dx, dev(res), dev(w), dev(b), 1, N, C)
+    es, eo, _, _ = oracle.fused_residual_layernorm_forward(x, res, w, b)
+    assert np.array_equal(dx.cpu().numpy(), es)
+    assert_close(out, eo, "fused ln out (in place)")
+
+
+# ------------------------------------------------------------------ matmul
+def mm_inputs(M, C, OC, seed, bias=True):
+    r = np.random.default_rng(seed)
+    x = r.standard_normal((M, C), dtype=np.float32)
+    w = r.standard_normal((OC, C), dtype=np.float32) * np.float32(0.02)
+    b = (r.standard_normal(OC, dtype=np.float32) * np.float32(0.02)) if bias else None
+    return x, w, b
+
+
+def run_matmul(x, w, b, gelu=None):
+    M, C = x.shape
+    OC = w.shape[0]
+    full, out, pad = guard((M, OC))
+    db = dev(b) if b is not None else None
+    if gelu is None:
+        g2.matmul_forward(out, dev(x), dev(w), db, 1, M, C, OC)
+    else:
+        g2.matmul_forward_gelu(out, dev(x), dev(w), db, 1, M, C, OC, gelu)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    return out
+
+
+@pytest.mark.parametrize("M,C,OC", [
+    (8192, 768, 2304), (8192, 768, 768), (8192, 768, 3072), (8192, 3072, 768),   # GPT-2 124M
+    (256, 768, 2304), (256, 3072, 768),                                          # B=4, T=64
+    (4096, 1024, 3072), (4096, 4096, 1024),                                      # GPT-2 350M
+    (128, 32, 192), (1, 4, 1), (130, 36, 200), (77, 100, 81), (300, 768, 50),    # edges
+])
+def test_matmul_bias(M, C, OC):
+    say(f"matmul M={M} C={C} OC={OC}")
+    x, w, b = mm_inputs(M, C, OC, 120)
+    out = run_matmul(x, w, b)
+    assert_close(out, oracle.matmul_forward(x, w, b), "matmul")
+
+
+def test_matmul_lm_head_no_bias():
+    # 768 -> 50257 without bias; the oracle runs on a row subset to stay in seconds,
+    # which is exact because rows are independent.
+    M, C, OC = 8192, 768, 50257
+    say(f"matmul lm-head M={M} C={C} OC={OC}")
+    x, w, _ = mm_inputs(M, C, OC, 121, bias=False)
+    out = run_matmul(x, w, None)
+    rows = np.r_[0:64, 4000:4064, 8128:8192]
+    exp = oracle.matmul_forward(x[rows], w, None)
+    assert_close(out[torch.from_numpy(rows).cuda()], exp, "lm-head rows")
+    # size-independent property over the full output: linearity in the input rows
+    # (row i + row j through the same weights) checked on a column subset in float64
+    got = out[:, ::997].cpu().numpy().astype(np.float64)
+    ref = x.astype(np.float64) @ w[::997].astype(np.float64).T
+    assert np.abs(got - ref).max() < 2e-5
+
+
+def test_matmul_generic_path_unaligned_k():
+    x, w, b = mm_inputs(33, 30, 17, 122)  # C % 4 != 0
+    assert_close(run_matmul(x, w, b), oracle.matmul_forward(x, w, b), "matmul generic")
+    assert_close(run_matmul(x, w, None), oracle.matmul_forward(x, w, None), "matmul generic nobias")
+
+
+@pytest.mark.parametrize("M,C,OC", [(8192, 768, 3072), (256, 768, 3072), (70, 64, 100)])
+def test_matmul_gelu_epilogue(M, C, OC):
+    say(f"matmul+gelu M={M} C={C} OC={OC}")
+    x, w, b = mm_inputs(M, C, OC, 123)
+    exp = oracle.matmul_forward(x, w, b)
+    assert_close(run_matmul(x, w, b, gelu=0), exp, "matmul is_gelu=0")
+    out = run_matmul(x, w, b, gelu=1)
+    # gelu has slope <= 1.13, so the matmul tolerance carries over to the composition
+    assert_close(out, oracle.gelu_forward(exp), "matmul is_gelu=1")
+
+
+def test_matmul_identity_weight():
+    M, C = 200, 192
+    r = np.random.default_rng(124)
+    x = r.standard_normal((M, C), dtype=np.float32)
+    b = r.standard_normal(C, dtype=np.float32)
+    out = run_matmul(x, np.eye(C, dtype=np.float32), b)
+    assert np.array_equal(out.cpu().numpy(), b[None, :] + x)
+
+
+# ------------------------------------------------------------------ attention
+@pytest.mark.parametrize("B,T,NH", [(8, 1024, 12), (8, 256, 12), (2, 1024, 16), (4, 256, 16),
+                                    (4, 64, 12), (1, 1, 2), (2, 33, 3), (1, 130, 2), (1, 200, 1)])
+def test_attention_hs64(B, T, NH):
+    say(f"attention B={B} T={T} NH={NH} HS=64")
+    C = NH * 64
+    qkv = np.random.default_rng(130).standard_normal((B, T, 3 * C), dtype=np.float32)
+    dq = dev(qkv)
+    full, out, pad = guard((B, T, C))
+    g2.attention_forward(out, None, None, dq, B, T, C, NH)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    assert np.array_equal(dq.cpu().numpy(), qkv), "attention must not write its input"
+    assert_close(out, oracle.attention_forward(qkv, NH), "attention")
+
+
+@pytest.mark.parametrize("B,T,NH,hs", [(2, 40, 4, 32), (1, 70, 2, 16), (1, 9, 3, 128), (2, 65, 2, 20)])
+def test_attention_other_head_sizes(B, T, NH, hs):
+    say(f"attention generic B={B} T={T} NH={NH} HS={hs}")
+    C = NH * hs
+    qkv = np.random.default_rng(131).standard_normal((B, T, 3 * C), dtype=np.float32)
+    out = torch.empty((B, T, C), device="cuda")
+    g2.attention_forward(out, None, None, dev(qkv), B, T, C, NH)
+    assert_close(out, oracle.attention_forward(qkv, NH), "attention generic")
+
+
+def test_attention_large_scores_stay_finite():
+    B, T, NH = 1, 160, 2
+    C = NH * 64
+    qkv = np.random.default_rng(132).standard_normal((B, T, 3 * C), dtype=np.float32)
+    qkv[..., :2 * C] *= 6.0  # scores of a few hundred: softmax is nearly one-hot
+    out = torch.empty((B, T, C), device="cuda")
+    g2.attention_forward(out, None, None, dev(qkv), B, T, C, NH)
+    assert_close(out, oracle.attention_forward(qkv, NH), "attention large scores")
+
+
+def test_attention_causality_bitwise():
+    B, T, NH = 1, 192, 2
+    C = NH * 64
+    qkv = np.random.default_rng(133).standard_normal((B, T, 3 * C), dtype=np.float32)
+    out1 = torch.empty((B, T, C), device="cuda")
+    out2 = torch.empty((B, T, C), device="cuda")
+    g2.attention_forward(out1, None, None, dev(qkv), B, T, C, NH)
+    qkv2 = qkv.copy()
+    qkv2[0, 100:] += 3.0
+    g2.attention_forward(out2, None, None, dev(qkv2), B, T, C, NH)
+    assert torch.equal(out1[0, :100], out2[0, :100])
+    assert not torch.equal(out1[0, 100:], out2[0, 100:])
+
+
+# ------------------------------------------------------------------ argmax
+@pytest.mark.parametrize("N,V", [(256, 50257), (3, 5), (17, 257), (4, 1)])
+def test_argmax_bit_exact(N, V):
+    say(f"argmax N={N} V={V}")
+    r = np.random.default_rng(140)
+    x = r.standard_normal((N, V), dtype=np.float32)
+    if V > 4:
+        x[0, 3] = x[0, V - 1] = 9.0   # tie: lowest index must win
+        x[1, :] = 1.5                 # all equal
+    full, ids, pad = guard((N,), torch.int32)
+    g2.argmax_forward(ids, dev(x), N, V)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    assert np.array_equal(ids.cpu().numpy(), oracle.argmax_forward(x))
+
+
+# ------------------------------------------------------------------ error paths
+def test_bad_shapes_raise_and_leave_the_device_usable():
+    a = torch.zeros(64, device="cuda")
+    with pytest.raises(g2.GPT2HipError):
+        g2.matmul_forward(a, a, a, None, 1, 1, 0, 8)
+    with pytest.raises(g2.GPT2HipError):
+        g2.attention_forward(a, None, None, a, 1, 4, 30, 4)
+    g2.residual_forward(a, a, a, 64)
+    torch.cuda.synchronize()
