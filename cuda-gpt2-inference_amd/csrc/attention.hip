@@ -272,8 +272,8 @@ int attention_forward_status(float* out, float* qkvr, float* att, const float* i
   (void)att;
   if (B < 0 || T < 0 || C < 1 || NH < 1 || C % NH != 0)
     return fail(GPT2HIP_EINVAL, "attention_forward: bad shape B=%d T=%d C=%d NH=%d", B, T, C, NH);
-  if (!out || !inp) return fail(GPT2HIP_EINVAL, "attention_forward: null pointer");
   if (B == 0 || T == 0) return GPT2HIP_OK;
+  if (!out || !inp) return fail(GPT2HIP_EINVAL, "attention_forward: null pointer");
   const int hs = C / NH;
   if (hs == HS && aligned16(inp) && aligned16(out)) {
     const int nqt = (T + BQ - 1) / BQ;

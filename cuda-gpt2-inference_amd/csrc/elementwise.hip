@@ -80,8 +80,8 @@ __global__ __launch_bounds__(kBlock) void map_scalar_kernel(float* out, const fl
 template <bool GELU>
 static int launch_map(const char* name, float* out, const float* inp1, const float* inp2, int N) {
   if (N < 0) return fail(GPT2HIP_EINVAL, "%s: N=%d", name, N);
-  if (!out || !inp1 || (!GELU && !inp2)) return fail(GPT2HIP_EINVAL, "%s: null pointer", name);
   if (N == 0) return GPT2HIP_OK;
+  if (!out || !inp1 || (!GELU && !inp2)) return fail(GPT2HIP_EINVAL, "%s: null pointer", name);
   const size_t n = (size_t)N;
   size_t done = 0;
   if (aligned16(out) && aligned16(inp1) && (GELU || aligned16(inp2))) {
@@ -164,9 +164,9 @@ int encoder_forward_status(float* out, const int* inp, const float* wte, const f
                            int T, int C) {
   using namespace g2;
   if (B < 0 || T < 0 || C < 1) return fail(GPT2HIP_EINVAL, "encoder_forward: bad shape B=%d T=%d C=%d", B, T, C);
-  if (!out || !inp || !wte || !wpe) return fail(GPT2HIP_EINVAL, "encoder_forward: null pointer");
   const size_t total = (size_t)B * T * C;
   if (total == 0) return GPT2HIP_OK;
+  if (!out || !inp || !wte || !wpe) return fail(GPT2HIP_EINVAL, "encoder_forward: null pointer");
   if (C % 4 == 0 && aligned16(out) && aligned16(wte) && aligned16(wpe)) {
     const size_t total4 = total / 4;
     hipLaunchKernelGGL(encoder_vec_kernel, dim3((unsigned)((total4 + kBlock - 1) / kBlock)),
@@ -205,8 +205,8 @@ void gelu_forward(float* out, const float* inp, int N) {
 int argmax_forward_status(int* ids, const float* logits, int N, int V) {
   using namespace g2;
   if (N < 0 || V < 1) return fail(GPT2HIP_EINVAL, "argmax_forward: bad shape N=%d V=%d", N, V);
-  if (!ids || !logits) return fail(GPT2HIP_EINVAL, "argmax_forward: null pointer");
   if (N == 0) return GPT2HIP_OK;
+  if (!ids || !logits) return fail(GPT2HIP_EINVAL, "argmax_forward: null pointer");
   hipLaunchKernelGGL(argmax_rows_kernel, dim3(N), dim3(kBlock), 0, 0, ids, logits, V);
   G2_LAUNCH_CHECK("argmax_forward");
   return GPT2HIP_OK;

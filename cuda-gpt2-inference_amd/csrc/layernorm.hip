@@ -124,12 +124,12 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
                             const float* bias, int B, int T, int C) {
   const char* name = FUSED ? "fused_residual_layernorm_forward" : "layernorm_forward";
   if (B < 0 || T < 0 || C < 1) return fail(GPT2HIP_EINVAL, "%s: bad shape B=%d T=%d C=%d", name, B, T, C);
-  if (!out || !inp1 || !weight || !bias || (FUSED && (!res_out || !inp2)))
-    return fail(GPT2HIP_EINVAL, "%s: null pointer", name);
   const long long N64 = (long long)B * T;
   if (N64 > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "%s: B*T too large", name);
   const int N = (int)N64;
   if (N == 0) return GPT2HIP_OK;
+  if (!out || !inp1 || !weight || !bias || (FUSED && (!res_out || !inp2)))
+    return fail(GPT2HIP_EINVAL, "%s: null pointer", name);
   const dim3 grid((N + kRowsPerBlock - 1) / kRowsPerBlock), block(kRowsPerBlock * kWave);
   const bool vec = (C % 4 == 0) && C <= 4096 && aligned16(out) && aligned16(inp1) &&
                    aligned16(weight) && aligned16(bias) &&

@@ -249,11 +249,11 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
                            int B, int T, int C, int OC, bool gelu) {
   if (B < 0 || T < 0 || C < 1 || OC < 1)
     return fail(GPT2HIP_EINVAL, "matmul_forward: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
-  if (!out || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward: null pointer");
   const long long M64 = (long long)B * T;
   if (M64 > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: B*T too large");
   const int M = (int)M64;
   if (M == 0) return GPT2HIP_OK;
+  if (!out || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward: null pointer");
   if (C % 4 != 0 || !aligned16(inp) || !aligned16(weight)) {
     const size_t total = (size_t)M * OC;
     hipLaunchKernelGGL(matmul_generic_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, 0,
