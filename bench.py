@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPT-2 fp32 forward pass on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one gpt2_forward over one batch of synthetic token ids (GPT-2 124M,
+B=8, T=1024, seeded random weights; ids already resident in HBM).  Prints ONE
+JSON line on stdout: whole-forward tokens/s, the roofline position of the
+dominant kernel (the FP32-MFMA GEMM) measured with HIP events around every
+launch of a second, identical set of K steps, the per-launch breakdown, the
+stand-alone kernel figures at the BASELINE shapes, and the CPU oracle timed on
+the host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
+PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def init_params_on_device(model, syn, cfg, seed):
+    """GPT-2 initialisation written straight into the device parameter buffer."""
+    import torch
+    flat = model.params_tensor()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    L = cfg["num_layers"]
+    off = 0
+    for name, shape in syn.param_shapes(**cfg).items():
+        n = int(math.prod(shape))
+        seg = flat[off:off + n]
+        if name in ("wte", "qkvw", "fcw"):
+            seg.normal_(0.0, 0.02, generator=g)
+        elif name in ("attprojw", "fcprojw"):
+            seg.normal_(0.0, 0.02 / math.sqrt(2 * L), generator=g)
+        elif name == "wpe":
+            seg.normal_(0.0, 0.01, generator=g)
+        elif name in ("ln1w", "ln2w", "lnfw"):
+            seg.fill_(1.0)
+        else:
+            seg.zero_()
+        off += n
+    assert off == flat.numel()
+
+
+def forward_flops(cfg, B, T):
+    C, L, V, NH = cfg["channels"], cfg["num_layers"], cfg["vocab_size"], cfg["num_heads"]
+    M = B * T
+    mm = {"matmul_qkv": 2 * M * C * 3 * C, "matmul_attproj": 2 * M * C * C,
+          "matmul_fc_gelu": 2 * M * C * 4 * C, "matmul_fcproj": 2 * M * 4 * C * C}
+    per_forward = {k: v * L for k, v in mm.items()}
+    per_forward["matmul_lmhead"] = 2 * M * C * V
+    per_forward["attention"] = L * 4 * B * NH * (C // NH) * T * (T + 1) // 2
+    return per_forward
+
+
+def forward_bytes(cfg, B, T):
+    C, L = cfg["channels"], cfg["num_layers"]
+    M = B * T
+    return {"encoder": 4 * M + 8 * M * C + 4 * T * C,
+            "layernorm": 8 * M * C + 8 * C,
+            "fused_residual_layernorm": 2 * L * (16 * M * C + 8 * C)}
+
+
+LAUNCHES = {"encoder": 1, "layernorm": 1, "matmul_lmhead": 1}
+
+
+def time_launch(g2, fn, iters=30, warmup=10):
+    """Median-free simple average: HIP events on the null stream around `iters` launches."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t = g2.Timer()
+    t.start()
+    for i in range(iters):
+        fn(warmup + i)
+    return t.stop_ms() / iters
+
+
+def standalone(g2):
+    """Per-kernel figures at the BASELINE shapes (configs 1-3)."""
+    import torch
+    out = []
+    M = 8192
+    dev = "cuda"
+    # fused residual+layernorm: rotate over 8 buffer sets (> 256 MiB Infinity Cache)
+    for C in (768, 1024):
+        sets = 8
+        x = torch.randn(sets, M, C, device=dev)
+        r = torch.randn(sets, M, C, device=dev)
+        o = torch.empty(sets, M, C, device=dev)
+        s = torch.empty(sets, M, C, device=dev)
+        mean = torch.empty(M, device=dev)
+        rstd = torch.empty(M, device=dev)
+        w = torch.randn(C, device=dev) * 0.1 + 1
+        b = torch.randn(C, device=dev) * 0.1
+        ms = time_launch(g2, lambda i: g2.fused_residual_layernorm_forward(
+            s[i % sets], o[i % sets], mean, rstd, x[i % sets], r[i % sets], w, b, 8, 1024, C),
+            iters=40, warmup=8)
+        nbytes = 16 * M * C + 8 * C + 8 * M
+        gbs = nbytes / ms / 1e6
+        out.append({"kernel": "fused_residual_layernorm", "shape": f"N={M},C={C}", "ms": ms,
+                    "GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
+                    "note": f"rotating {sets} buffer sets, {sets * 4 * M * C * 4 >> 20} MiB"})
+        del x, r, o, s
+    # matmul at the GPT-2 124M linear shapes
+    for (C, OC, bias) in ((768, 2304, True), (768, 768, True), (768, 3072, True), (3072, 768, True),
+                          (768, 50257, False)):
+        x = torch.randn(M, C, device=dev)
+        w = torch.randn(OC, C, device=dev) * 0.02
+        bb = torch.randn(OC, device=dev) * 0.02 if bias else None
+        o = torch.empty(M, OC, device=dev)
+        ms = time_launch(g2, lambda i: g2.matmul_forward(o, x, w, bb, 8, 1024, C, OC),
+                         iters=10 if OC > 10000 else 20)
+        tf = 2.0 * M * C * OC / ms / 1e9
+        out.append({"kernel": "matmul_forward", "shape": f"M={M},C={C},OC={OC}", "ms": ms,
+                    "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS})
+        del x, w, o
+    # causal attention
+    for (B, T, NH) in ((8, 1024, 12), (8, 256, 12), (8, 1024, 16), (8, 256, 16)):
+        C = NH * 64
+        qkv = torch.randn(B, T, 3 * C, device=dev)
+        o = torch.empty(B, T, C, device=dev)
+        ms = time_launch(g2, lambda i: g2.attention_forward(o, None, None, qkv, B, T, C, NH))
+        tf = 4.0 * B * NH * 64 * T * (T + 1) / 2 / ms / 1e9
+        out.append({"kernel": "attention_forward", "shape": f"B={B},T={T},NH={NH},HS=64", "ms": ms,
+                    "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS})
+        del qkv, o
+    # the other bandwidth kernels at the 124M B=8 T=1024 sizes
+    N = M * 3072
+    a = torch.randn(4, N, device=dev)
+    o = torch.empty(4, N, device=dev)
+    ms = time_launch(g2, lambda i: g2.gelu_forward(o[i % 4], a[i % 4], N))
+    out.append({"kernel": "gelu_forward", "shape": f"N={N}", "ms": ms, "GB/s": 8 * N / ms / 1e6,
+                "frac_hbm": 8 * N / ms / 1e6 / PEAK_HBM_GBS})
+    N = M * 768
+    ms = time_launch(g2, lambda i: g2.residual_forward(o[i % 4][:N], a[i % 4][:N], a[(i + 1) % 4][:N], N))
+    out.append({"kernel": "residual_forward", "shape": f"N={N}", "ms": ms, "GB/s": 12 * N / ms / 1e6,
+                "frac_hbm": 12 * N / ms / 1e6 / PEAK_HBM_GBS})
+    del a, o
+    for C in (768,):
+        x = torch.randn(8, M, C, device=dev)
+        o = torch.empty(8, M, C, device=dev)
+        w = torch.ones(C, device=dev)
+        b = torch.zeros(C, device=dev)
+        ms = time_launch(g2, lambda i: g2.layernorm_forward(o[i % 8], None, None, x[i % 8], w, b, 8,
+                                                            1024, C), iters=40, warmup=8)
+        nb = 8 * M * C + 8 * C
+        out.append({"kernel": "layernorm_forward", "shape": f"N={M},C={C}", "ms": ms,
+                    "GB/s": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS})
+    return out
+
+
+def cpu_baseline(model, cfg, B, T):
+    """The CPU oracle on the host cores: one forward of the whole benchmark batch
+    (a few seconds on 16 cores), after one untimed pass at B=1 to warm the threads."""
+    import numpy as np
+    import oracle
+    params = model.params_tensor().cpu().numpy()
+    ids = np.random.default_rng(0).integers(0, cfg["vocab_size"], (B, T), dtype=np.int32)
+    kw = dict(maxT=cfg["max_seq_len"], V=cfg["vocab_size"], L=cfg["num_layers"],
+              NH=cfg["num_heads"], C=cfg["channels"])
+    oracle.gpt2_forward(params, ids[:1], **kw)
+    t0 = time.monotonic()
+    oracle.gpt2_forward(params, ids, **kw)
+    dt = time.monotonic() - t0
+    return {"value": B * T / dt, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"one forward of the same workload, B={B}, T={T} ({dt:.2f} s wall); "
+                      "plain-C/OpenMP restatement of llm.c's CPU gpt2_forward"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--model", choices=("124M", "350M"), default="124M")
+    ap.add_argument("--batch", type=int, default=None)
+    ap.add_argument("--no-standalone", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (the forward pass shards over the batch with "
+              "no exchange, so N GPUs would be N independent copies of this run); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    g2 = importlib.import_module("cuda-gpt2-inference_amd")
+    syn = importlib.import_module("cuda-gpt2-inference_amd.synthetic")
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+
+    cfg = dict(g2.GPT2_124M if args.model == "124M" else g2.GPT2_350M)
+    B = args.batch or (8 if args.model == "124M" else 4)
+    T = 1024
+    model = g2.GPT2(**cfg)
+    init_params_on_device(model, syn, cfg, seed=1337)
+    ids = torch.randint(0, cfg["vocab_size"], (B, T), dtype=torch.int32, device="cuda")
+    model.reserve(B, T)
+
+    for _ in range(args.warmup):
+        model.forward(ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.forward(ids)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tokens_per_s = B * T * args.steps / dt
+    finite = bool(torch.isfinite(model.logits()[0, :4]).all())
+    log(f"forward {args.model} B={B} T={T}: {ms_per_step:.3f} ms/step, {tokens_per_s:,.0f} tok/s"
+        f" (logits finite: {finite})")
+
+    # the same K steps again with a HIP event around every launch
+    prof = {k: 0.0 for k in g2.PROF_CATEGORIES}
+    for _ in range(args.steps):
+        for k, v in model.forward_profiled(ids).items():
+            prof[k] += v
+    prof = {k: v / args.steps for k, v in prof.items()}   # ms per forward per category
+    flops = forward_flops(cfg, B, T)
+    nbytes = forward_bytes(cfg, B, T)
+    L = cfg["num_layers"]
+    kernels = []
+    for k in g2.PROF_CATEGORIES:
+        launches = LAUNCHES.get(k, 2 * L if k == "fused_residual_layernorm" else L)
+        row = {"launch": k, "launches_per_forward": launches, "ms_per_forward": prof[k],
+               "ms_per_launch": prof[k] / launches}
+        if k in flops:
+            tf = flops[k] / prof[k] / 1e9
+            row.update({"TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS})
+        else:
+            gbs = nbytes[k] / prof[k] / 1e6
+            row.update({"GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
+                        "note": "inside the forward pass, operands may be served by the 256 MiB "
+                                "Infinity Cache"})
+        kernels.append(row)
+        log(f"  {k:26s} {prof[k]:8.3f} ms/fwd  " + (f"{row.get('TFLOP/s', 0):7.1f} TFLOP/s"
+            if k in flops else f"{row.get('GB/s', 0):7.0f} GB/s"))
+    # dominant kernel: the bias (non-GELU) instantiation of the MFMA GEMM
+    dom = ("matmul_qkv", "matmul_attproj", "matmul_fcproj", "matmul_lmhead")
+    dom_launches = 3 * L + 1
+    dom_flops = sum(flops[k] for k in dom) / dom_launches
+    dom_ms = sum(prof[k] for k in dom) / dom_launches
+    achieved = dom_flops / dom_ms / 1e9
+    roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                "kernel": "matmul_mfma_kernel<128,192,4,2,false>",
+                "avg_launch_ms": dom_ms, "flops_per_launch": dom_flops,
+                "launches_per_forward": dom_launches}
+
+    result = {
+        "metric": "GPT-2 124M fp32 fwd tokens/s (B=8,T=1024); matmul % FP32 MFMA peak",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"GPT-2 {args.model} fp32 forward, B={B}, T={T}, seeded random "
+                               "weights, uniform random token ids resident in HBM",
+                   "global_batch": B, "seq_len": T},
+        "roofline": roofline,
+        "forward_frac_fp32_mfma": (sum(flops.values()) / (ms_per_step * 1e9)) / PEAK_FP32_MFMA_TFLOPS,
+        "kernels": kernels,
+    }
+    if not args.no_standalone:
+        result["standalone"] = standalone(g2)
+        for r in result["standalone"]:
+            log("  standalone", json.dumps(r))
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(model, cfg, B, T)
+        log("  cpu_baseline", json.dumps(result["cpu_baseline"]))
+    model.close()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -40,7 +40,7 @@ EXPORTS = (
     "argmax_forward", "argmax_forward_status",
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
-    "gpt2_forward_device_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
+    "gpt2_forward_device_status", "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
     "gpt2hip_timer_stop_ms",
 )
@@ -66,6 +66,10 @@ class GPT2Config(ctypes.Structure):
                 ("num_layers", ctypes.c_int), ("num_heads", ctypes.c_int),
                 ("channels", ctypes.c_int)]
 
+
+# order of the GPT2_PROF_* enum in the header
+PROF_CATEGORIES = ("encoder", "layernorm", "matmul_qkv", "attention", "matmul_attproj",
+                   "fused_residual_layernorm", "matmul_fc_gelu", "matmul_fcproj", "matmul_lmhead")
 
 GPT2_124M = dict(max_seq_len=1024, vocab_size=50257, num_layers=12, num_heads=12, channels=768)
 GPT2_350M = dict(max_seq_len=1024, vocab_size=50257, num_layers=24, num_heads=16, channels=1024)
@@ -110,6 +114,8 @@ def lib() -> ctypes.CDLL:
         L.gpt2_forward_status.argtypes, L.gpt2_forward_status.restype = [vp, vp, ci, ci], ci
         L.gpt2_forward_device_status.argtypes = [vp, vp, ci, ci]
         L.gpt2_forward_device_status.restype = ci
+        L.gpt2_forward_profiled_status.argtypes = [vp, vp, ci, ci, ctypes.POINTER(ctypes.c_float)]
+        L.gpt2_forward_profiled_status.restype = ci
         L.gpt2_logits.argtypes, L.gpt2_logits.restype = [vp], vp
         L.gpt2_lnf.argtypes, L.gpt2_lnf.restype = [vp], vp
         L.gpt2_argmax_status.argtypes, L.gpt2_argmax_status.restype = [vp, vp], ci
@@ -265,6 +271,15 @@ class GPT2:
         else:
             _check(lib().gpt2_forward_device_status(self._h, _i32(inputs), B, T), "gpt2_forward")
         self._shape = (B, T)
+
+    def forward_profiled(self, inputs_device):
+        """Forward with per-launch HIP events; returns {category: ms} for this pass."""
+        B, T = inputs_device.shape
+        ms = (ctypes.c_float * len(PROF_CATEGORIES))()
+        _check(lib().gpt2_forward_profiled_status(self._h, _i32(inputs_device), B, T, ms),
+               "gpt2_forward_profiled")
+        self._shape = (B, T)
+        return dict(zip(PROF_CATEGORIES, (float(x) for x in ms)))
 
     def logits(self):
         B, T = self._shape

@@ -88,44 +88,70 @@ static int reserve(GPT2* m, int B, int T) {
   return GPT2HIP_OK;
 }
 
+// Optional per-launch timing: an event is recorded on the null stream before the
+// first launch and after every launch; category[i] names the launch between
+// events i and i+1.
+struct Profile {
+  std::vector<hipEvent_t> events;
+  std::vector<int> category;
+  int mark(int cat) {  // cat < 0: the opening event
+    hipEvent_t e;
+    G2_HIP(hipEventCreate(&e));
+    events.push_back(e);
+    if (cat >= 0) category.push_back(cat);
+    G2_HIP(hipEventRecord(e, 0));
+    return GPT2HIP_OK;
+  }
+  ~Profile() {
+    for (hipEvent_t e : events) (void)hipEventDestroy(e);
+  }
+};
+
 // The forward pass proper; ids are already in m->ids.
-static int forward_resident(GPT2* m, int B, int T) {
+static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr) {
   const GPT2Config& c = m->cfg;
   const int C = c.channels, L = c.num_layers, NH = c.num_heads, V = c.vocab_size;
   const size_t cs = (size_t)C;
   auto P = [&](int which) { return m->params + m->param_off[which]; };
-#define G2_TRY(call)          \
-  do {                        \
+#define G2_TRY(call)                  \
+  do {                                \
     if (int rc_ = (call)) return rc_; \
   } while (0)
+#define G2_STEP(cat, call)                \
+  do {                                    \
+    G2_TRY(call);                         \
+    if (prof) G2_TRY(prof->mark(cat));    \
+  } while (0)
+  if (prof) G2_TRY(prof->mark(-1));
 
   float* residual = m->res_a;  // current residual stream
   float* other = m->res_b;
-  G2_TRY(encoder_forward_status(residual, m->ids, P(P_WTE), P(P_WPE), B, T, C));
+  G2_STEP(GPT2_PROF_ENCODER, encoder_forward_status(residual, m->ids, P(P_WTE), P(P_WPE), B, T, C));
   // the one stand-alone layernorm: ln1 of layer 0
-  G2_TRY(layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, T, C));
+  G2_STEP(GPT2_PROF_LAYERNORM, layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, T, C));
   for (int l = 0; l < L; l++) {
-    G2_TRY(matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
+    G2_STEP(GPT2_PROF_MATMUL_QKV, matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
                                  B, T, C, 3 * C));
-    G2_TRY(attention_forward_status(m->atty, nullptr, nullptr, m->qkv, B, T, C, NH));
-    G2_TRY(matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs,
+    G2_STEP(GPT2_PROF_ATTENTION, attention_forward_status(m->atty, nullptr, nullptr, m->qkv, B, T, C, NH));
+    G2_STEP(GPT2_PROF_MATMUL_ATTPROJ, matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs,
                                  P(P_ATTPROJB) + l * cs, B, T, C, C));
     // residual2 = residual + attproj ; ln = ln2(residual2)
-    G2_TRY(fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual,
+    G2_STEP(GPT2_PROF_FUSED_RESIDUAL_LAYERNORM, fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual,
                                                    m->proj, P(P_LN2W) + l * cs, P(P_LN2B) + l * cs,
                                                    B, T, C));
-    G2_TRY(matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs,
+    G2_STEP(GPT2_PROF_MATMUL_FC_GELU, matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs,
                                       P(P_FCB) + l * 4 * cs, B, T, C, 4 * C, 1));
-    G2_TRY(matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
+    G2_STEP(GPT2_PROF_MATMUL_FCPROJ, matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
                                  P(P_FCPROJB) + l * cs, B, T, 4 * C, C));
     // residual3 = residual2 + fcproj ; ln = ln1 of the next layer, or the final layernorm
     const float* nw = (l + 1 < L) ? P(P_LN1W) + (l + 1) * cs : P(P_LNFW);
     const float* nb = (l + 1 < L) ? P(P_LN1B) + (l + 1) * cs : P(P_LNFB);
-    G2_TRY(fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other,
+    G2_STEP(GPT2_PROF_FUSED_RESIDUAL_LAYERNORM, fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other,
                                                    m->proj, nw, nb, B, T, C));
   }
   // lm-head: weight-tied to wte, no bias, unpadded vocabulary
-  G2_TRY(matmul_forward_status(m->logits, m->ln, P(P_WTE), nullptr, B, T, C, V));
+  G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_status(m->logits, m->ln, P(P_WTE), nullptr, B, T, C, V));
+#undef G2_STEP
 #undef G2_TRY
   m->last_B = B;
   m->last_T = T;
@@ -214,6 +240,26 @@ int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int
   G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
                         hipMemcpyDeviceToDevice, 0));
   return forward_resident(model, B, T);
+}
+
+int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, int T,
+                                 float* ms_per_category) {
+  using namespace g2;
+  if (int rc = reserve(model, B, T)) return rc;
+  if (!inputs_device || !ms_per_category)
+    return fail(GPT2HIP_EINVAL, "gpt2_forward_profiled: null pointer");
+  G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
+                        hipMemcpyDeviceToDevice, 0));
+  Profile prof;
+  if (int rc = forward_resident(model, B, T, &prof)) return rc;
+  G2_HIP(hipEventSynchronize(prof.events.back()));
+  for (int i = 0; i < GPT2_PROF_COUNT; i++) ms_per_category[i] = 0.f;
+  for (size_t i = 0; i < prof.category.size(); i++) {
+    float ms = 0.f;
+    G2_HIP(hipEventElapsedTime(&ms, prof.events[i], prof.events[i + 1]));
+    ms_per_category[prof.category[i]] += ms;
+  }
+  return GPT2HIP_OK;
 }
 
 const float* gpt2_logits(const GPT2* model) { return model ? model->logits : nullptr; }

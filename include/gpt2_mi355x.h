@@ -143,6 +143,24 @@ int gpt2_reserve(GPT2* model, int B, int T);
 int gpt2_forward_status(GPT2* model, const int* inputs_host, int B, int T);
 void gpt2_forward(GPT2* model, const int* inputs_host, int B, int T);
 int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int T);
+/* The same forward pass with a HIP event recorded on the null stream around
+ * every launch; waits for completion and adds each launch's elapsed ms into
+ * ms_per_category[GPT2_PROF_COUNT] (host memory).  No counterpart in the
+ * reference, whose timings come from an external profiler (README.md:179). */
+enum {
+  GPT2_PROF_ENCODER = 0,
+  GPT2_PROF_LAYERNORM,
+  GPT2_PROF_MATMUL_QKV,
+  GPT2_PROF_ATTENTION,
+  GPT2_PROF_MATMUL_ATTPROJ,
+  GPT2_PROF_FUSED_RESIDUAL_LAYERNORM,
+  GPT2_PROF_MATMUL_FC_GELU,
+  GPT2_PROF_MATMUL_FCPROJ,
+  GPT2_PROF_MATMUL_LMHEAD,
+  GPT2_PROF_COUNT
+};
+int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, int T,
+                                 float* ms_per_category);
 const float* gpt2_logits(const GPT2* model);
 /* Final layernorm output (B,T,C) of the last forward, on the device. */
 const float* gpt2_lnf(const GPT2* model);
