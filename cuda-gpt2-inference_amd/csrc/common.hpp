@@ -83,11 +83,16 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// tanh-GELU, the formula of reference 9_matmul_async_cg_tf32_gelu.cuh:5-11.
+// tanh-GELU, 0.5x(1+tanh(u)) with u = sqrt(2/pi)(x + 0.044715x^3), the formula of
+// reference 9_matmul_async_cg_tf32_gelu.cuh:5-11, evaluated through the identity
+// 0.5(1+tanh(u)) = 1/(1+exp(-2u)): one hardware exp2 and one reciprocal, and no
+// cancellation in 1+tanh(u) for negative x.
 __device__ __forceinline__ float gelu_tanh(float x) {
-  const float k = 0.7978845608028654f;  // sqrtf(2/pi)
-  const float cube = 0.044715f * x * x * x;
-  return 0.5f * x * (1.0f + tanhf(k * (x + cube)));
+  const float k = 0.7978845608028654f;            // sqrt(2/pi)
+  const float c = -2.0f * 1.4426950408889634f * k;  // -2 log2(e) sqrt(2/pi)
+  const float u = x + 0.044715f * x * x * x;
+  const float e = __builtin_amdgcn_exp2f(c * u);  // exp(-2u); +inf for very negative x
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 #endif
 

@@ -5,8 +5,9 @@
 // Tiling.  A workgroup owns a BM x BN output tile and walks K in slabs of
 // BK = 32.  Both operands are K-contiguous in memory ("NT" GEMM), so a slab of
 // either is rows of 32 floats = 8 chunks of 16 bytes.  Slabs are fetched with
-// 128-bit global loads into registers one slab ahead, then stored to one of
-// two LDS buffers; one barrier per slab.  In LDS, chunk c of row r sits at
+// 128-bit global loads into registers two slabs ahead, then stored to one of
+// two LDS buffers; one barrier per slab, placed inside the slab's MFMA work so
+// that no wave waits on a store->barrier->read chain.  In LDS, chunk c of row r sits at
 // chunk position c ^ (r & 7): eight lanes that read the same logical chunk of
 // eight consecutive rows then hit eight different 16-byte bank groups, which
 // makes both the 128-bit stores and the 128-bit operand reads conflict-free.
@@ -48,7 +49,7 @@ __device__ __forceinline__ void tile_of_block(int pid, int ntm, int ntn, int& tm
   }
 }
 
-template <int BM, int BN, int WGM, int WGN, bool GELU>
+template <int BM, int BN, int WGM, int WGN, bool GELU, bool KTAIL>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
     const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn) {
@@ -72,7 +73,11 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
   const int m0 = tm * BM, n0 = tn * BN;
 
   // ---- global -> register staging --------------------------------------
-  // chunk q = tid + j*NT of the slab: row q/8, chunk q%8.
+  // chunk q = tid + j*NT of the slab: row q/8, chunk q%8.  Rows past the end of the
+  // matrix are clamped to its last row: they produce accumulator rows / columns
+  // that the epilogue never stores, so M and N edges need no masking.  Only a K
+  // tail (K % 32 != 0, KTAIL) must contribute zeros; that fill is applied when
+  // the registers are stored to LDS, a slab after the loads were issued.
   const float* a_src[A_PER];
   const float* b_src[B_PER];
   int a_dst[A_PER], b_dst[B_PER];
@@ -81,41 +86,33 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
   for (int j = 0; j < A_PER; j++) {
     const int q = tid + j * NT;
     const int r = q >> 3, c = q & 7;
-    const int gm = m0 + r;
-    a_src[j] = (gm < M) ? inp + (size_t)gm * K + kc : nullptr;
+    a_src[j] = inp + (size_t)min(m0 + r, M - 1) * K;
     a_dst[j] = r * CHUNKS + (c ^ (r & 7));
   }
 #pragma unroll
   for (int j = 0; j < B_PER; j++) {
     const int q = tid + j * NT;
     const int r = q >> 3, c = q & 7;
-    const int gn = n0 + r;
-    b_src[j] = (gn < N) ? weight + (size_t)gn * K + kc : nullptr;
+    b_src[j] = weight + (size_t)min(n0 + r, N - 1) * K;
     b_dst[j] = BM * CHUNKS + r * CHUNKS + (c ^ (r & 7));
   }
 
   f32x4 a_reg[A_PER], b_reg[B_PER];
+  bool reg_kin = true;  // whether the chunk held in the registers lies inside K
   auto fetch = [&](int k0) {
-    const bool kin = (k0 + kc) < K;  // K is a multiple of 4: a chunk is all in or all out
+    reg_kin = (k0 + kc) < K;  // K is a multiple of 4: a chunk is all in or all out
+    const int ko = reg_kin ? k0 + kc : 0;  // past the end: re-read a valid address
 #pragma unroll
-    for (int j = 0; j < A_PER; j++) {
-      f32x4 z = {0.f, 0.f, 0.f, 0.f};
-      if (kin && a_src[j]) z = *reinterpret_cast<const f32x4*>(a_src[j] + k0);
-      a_reg[j] = z;
-    }
+    for (int j = 0; j < A_PER; j++) a_reg[j] = *reinterpret_cast<const f32x4*>(a_src[j] + ko);
 #pragma unroll
-    for (int j = 0; j < B_PER; j++) {
-      f32x4 z = {0.f, 0.f, 0.f, 0.f};
-      if (kin && b_src[j]) z = *reinterpret_cast<const f32x4*>(b_src[j] + k0);
-      b_reg[j] = z;
-    }
+    for (int j = 0; j < B_PER; j++) b_reg[j] = *reinterpret_cast<const f32x4*>(b_src[j] + ko);
   };
-  auto stash = [&](int buf) {
-    f32x4* s = lds + buf * STAGE;
+  auto stash = [&](f32x4* s) {
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < A_PER; j++) s[a_dst[j]] = a_reg[j];
+    for (int j = 0; j < A_PER; j++) s[a_dst[j]] = (!KTAIL || reg_kin) ? a_reg[j] : zero;
 #pragma unroll
-    for (int j = 0; j < B_PER; j++) s[b_dst[j]] = b_reg[j];
+    for (int j = 0; j < B_PER; j++) s[b_dst[j]] = (!KTAIL || reg_kin) ? b_reg[j] : zero;
   };
 
   // ---- accumulators, initialised with the bias of the lane's column ----
@@ -140,51 +137,121 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
 #pragma unroll
   for (int j = 0; j < TN; j++) b_row[j] = BM * CHUNKS + (wn * WN + j * 32 + (lane & 31)) * CHUNKS;
 
+  // Operands of k-group g (k = 8g .. 8g+7 of the slab) into register set p.
+  f32x4 af[2][TM], bf[2][TN];
+  auto read_ops = [&](const f32x4* buf, int g, int p) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) af[p][i] = buf[a_row[i] + ((2 * g + h) ^ sw)];
+#pragma unroll
+    for (int j = 0; j < TN; j++) bf[p][j] = buf[b_row[j] + ((2 * g + h) ^ sw)];
+  };
+  auto mfma_group = [&](int p) {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] =
+              __builtin_amdgcn_mfma_f32_32x32x2f32(af[p][i][e], bf[p][j][e], acc[i][j], 0, 0, 0);
+  };
+  // Scheduling groups: an MFMA occupies the matrix pipe for 64 cycles but issues in a
+  // few, so every LDS / global / VALU instruction of the loop is placed in the shadow
+  // of an MFMA instead of between two bursts of them.
+#define G2_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define G2_MFMA 0x008
+#define G2_VMEM_RD 0x020
+#define G2_DS_RD 0x100
+#define G2_DS_WR 0x200
+
+  // Software pipeline over slabs s = 0 .. nslab-1 (two LDS buffers, cur / nxt).  The
+  // body is branch-free: past the last slab it stores zeros to the idle buffer and
+  // re-reads a valid address, which nobody consumes.
+  //   group 0: MFMAs of group 0, reading group 1's operands
+  //   group 1: MFMAs of group 1, reading group 2's operands
+  //   group 2: MFMAs of group 2, reading group 3's operands and storing the
+  //            prefetched slab s+1 into nxt (whose last reads completed before the
+  //            previous barrier)
+  //            BARRIER (all cur reads complete; all nxt stores visible)
+  //   group 3: MFMAs of group 3, reading group 0 of slab s+1 from nxt and issuing
+  //            the global loads of slab s+2
+  // so the store->barrier->read chain never sits between two MFMAs with nothing to
+  // cover it, and global loads have a full slab of MFMA time to land.
   const int nslab = (K + BK - 1) / BK;
   fetch(0);
-  stash(0);
+  stash(lds);
+  fetch(BK);
   __syncthreads();
+  read_ops(lds, 0, 0);
 
   for (int s = 0; s < nslab; s++) {
     const f32x4* cur = lds + (s & 1) * STAGE;
-    if (s + 1 < nslab) fetch((s + 1) * BK);
+    f32x4* nxt = lds + ((s + 1) & 1) * STAGE;
 
-    f32x4 af[2][TM], bf[2][TN];
+    read_ops(cur, 1, 1);
+    mfma_group(0);
+    read_ops(cur, 2, 0);
+    mfma_group(1);
+    read_ops(cur, 3, 1);
+    stash(nxt);
+    mfma_group(0);
 #pragma unroll
-    for (int i = 0; i < TM; i++) af[0][i] = cur[a_row[i] + ((0 + h) ^ sw)];
+    for (int g = 0; g < 2; g++) {
 #pragma unroll
-    for (int j = 0; j < TN; j++) bf[0][j] = cur[b_row[j] + ((0 + h) ^ sw)];
-#pragma unroll
-    for (int g = 0; g < CHUNKS / 2; g++) {
-      const int p = g & 1;
-      if (g + 1 < CHUNKS / 2) {
-#pragma unroll
-        for (int i = 0; i < TM; i++) af[p ^ 1][i] = cur[a_row[i] + ((2 * (g + 1) + h) ^ sw)];
-#pragma unroll
-        for (int j = 0; j < TN; j++) bf[p ^ 1][j] = cur[b_row[j] + ((2 * (g + 1) + h) ^ sw)];
+      for (int i = 0; i < TM + TN; i++) {
+        G2_SGB(G2_MFMA, 1);
+        G2_SGB(G2_DS_RD, 1);
       }
-#pragma unroll
-      for (int e = 0; e < 4; e++)
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[p][i][e], bf[p][j][e], acc[i][j], 0,
-                                                             0, 0);
+      G2_SGB(G2_MFMA, 4 * TM * TN - (TM + TN));
     }
+#pragma unroll
+    for (int i = 0; i < TM + TN; i++) {
+      G2_SGB(G2_MFMA, 1);
+      G2_SGB(G2_DS_RD, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < A_PER + B_PER; i++) {
+      G2_SGB(G2_MFMA, 1);
+      G2_SGB(G2_DS_WR, 1);
+    }
+    G2_SGB(G2_MFMA, 4 * TM * TN - (TM + TN) - (A_PER + B_PER));
 
-    if (s + 1 < nslab) stash((s + 1) & 1);
     __syncthreads();
+
+    read_ops(nxt, 0, 0);
+    fetch((s + 2) * BK);
+    mfma_group(1);
+#pragma unroll
+    for (int i = 0; i < TM + TN; i++) {
+      G2_SGB(G2_MFMA, 1);
+      G2_SGB(G2_DS_RD, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < A_PER + B_PER; i++) {
+      G2_SGB(G2_MFMA, 1);
+      G2_SGB(G2_VMEM_RD, 1);
+    }
+    G2_SGB(G2_MFMA, 4 * TM * TN - (TM + TN) - (A_PER + B_PER));
   }
+#undef G2_SGB
 
   // ---- epilogue -----------------------------------------------------------
+  const bool full = (m0 + BM <= M) && (n0 + BN <= N);
 #pragma unroll
   for (int i = 0; i < TM; i++) {
 #pragma unroll
     for (int j = 0; j < TN; j++) {
       const int col = n0 + wn * WN + j * 32 + (lane & 31);
       const int rbase = m0 + wm * WM + i * 32 + 4 * h;
-      if (col < N) {
+      float* o = out + (size_t)rbase * N + col;
+      if (full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          float r = acc[i][j][v];
+          if (GELU) r = gelu_tanh(r);
+          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
+        }
+      } else if (col < N) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           const int row = rbase + 8 * (v >> 2) + (v & 3);
@@ -223,8 +290,11 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
   const long long tiles = (long long)ntm * ntn;
   if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
-  auto kfn = gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true>
-                  : matmul_mfma_kernel<BM, BN, WGM, WGN, false>;
+  const bool ktail = (K % BK) != 0;
+  auto kfn = ktail ? (gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true, true>
+                           : matmul_mfma_kernel<BM, BN, WGM, WGN, false, true>)
+                   : (gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true, false>
+                           : matmul_mfma_kernel<BM, BN, WGM, WGN, false, false>);
   static thread_local int configured_for = -1;  // device whose attribute was set (per variant)
   static thread_local int configured_mask = 0;
   int dev = 0;
@@ -233,7 +303,7 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
     configured_for = dev;
     configured_mask = 0;
   }
-  const int bit = gelu ? 2 : 1;
+  const int bit = (gelu ? 2 : 1) << (ktail ? 2 : 0);
   if (!(configured_mask & bit)) {
     G2_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
