@@ -266,6 +266,208 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Main kernel for K % 32 == 0 (every GPT-2 shape): same tiling, LDS layout and
+// MFMA mapping as above, but the K slabs go from global memory straight into LDS
+// with global_load_lds_dwordx4 (no staging registers, no ds_write, no per-slab
+// address arithmetic), and a wave owns a larger register tile so that fewer LDS
+// reads are needed per MFMA.  On this chip every non-MFMA instruction a SIMD
+// issues takes issue cycles away from the matrix pipe (measured: ~4 cycles per
+// VALU or ds_read, more per ds_write / global load), so the loop is built to
+// contain almost nothing but MFMAs: per wave and slab 24*TM*TN/... MFMAs,
+// 4*(TM+TN) ds_read_b128, (BM+BN)/8/waves LDS-DMA loads and 2*4 address updates.
+//
+// An LDS-DMA load writes lane l's 16 bytes to LDS address M0 + 16*l, i.e. one
+// instruction fills 8 consecutive 128-byte rows of a buffer.  The XOR chunk
+// swizzle is therefore applied on the global side: lane l (row l/8 of the group,
+// chunk position l%8) fetches logical chunk (l%8) ^ (l/8) of its row.
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void glb_void_t;
+
+template <int BM, int BN, int WGM, int WGN, bool GELU>
+__global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
+    float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
+    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn) {
+  constexpr int NW = WGM * WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int GROUPS = (BM + BN) / 8;  // 8-row groups per buffer, one DMA each
+  constexpr int DMA_PER = GROUPS / NW;   // DMAs per wave and slab
+  static_assert(GROUPS % NW == 0 && BM % 8 == 0, "tile/waves mismatch");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be 32x32 MFMA tiles");
+  constexpr int STAGE = (BM + BN) * CHUNKS;  // f32x4 per LDS buffer
+  constexpr int STAGE_BYTES = STAGE * 16;
+  constexpr int MFMAS = 4 * TM * TN;  // per k-group of 8
+
+  extern __shared__ f32x4 lds[];  // [2][STAGE]: A rows then B rows
+  char* const lds_bytes = reinterpret_cast<char*>(lds);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, ntm, ntn, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // ---- LDS-DMA descriptors -------------------------------------------------
+  // DMA j of this wave fills group gi = wave*DMA_PER + j (rows 8*gi .. 8*gi+7 of the
+  // buffer).  Rows past the end of a matrix are clamped to its last row: they only
+  // feed accumulator rows / columns that the epilogue does not store.
+  const char* dma_base[DMA_PER];  // wave-uniform: the tile's first row of A or of B
+  unsigned dma_off[DMA_PER];      // per lane: byte offset of its 16-byte chunk
+  {
+    const int rr = lane >> 3, c = (lane & 7) ^ rr;
+#pragma unroll
+    for (int j = 0; j < DMA_PER; j++) {
+      const int row = 8 * (wave * DMA_PER + j) + rr;
+      if (8 * (wave * DMA_PER + j) < BM) {
+        dma_base[j] = reinterpret_cast<const char*>(inp + (size_t)m0 * K);
+        dma_off[j] = (unsigned)((min(m0 + row, M - 1) - m0) * K + c * 4) * 4u;
+      } else {
+        dma_base[j] = reinterpret_cast<const char*>(weight + (size_t)n0 * K);
+        dma_off[j] = (unsigned)((min(n0 + row - BM, N - 1) - n0) * K + c * 4) * 4u;
+      }
+    }
+  }
+  const int nslab = K / BK;
+  auto dma_slab = [&](int slab, int buf) {
+    const size_t kbytes = (size_t)min(slab, nslab - 1) * (BK * 4);  // past the end: reload
+#pragma unroll
+    for (int j = 0; j < DMA_PER; j++)
+      __builtin_amdgcn_global_load_lds(
+          (glb_void_t*)(dma_base[j] + kbytes + dma_off[j]),
+          (lds_void_t*)(lds_bytes + buf * STAGE_BYTES + (wave * DMA_PER + j) * 1024), 16, 0, 0);
+  };
+
+  // ---- accumulators, initialised with the bias of the lane's column ----
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int col = n0 + wn * WN + j * 32 + (lane & 31);
+    const float bv = (bias != nullptr && col < N) ? bias[col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = bv;
+  }
+
+  // ---- operand read addresses: one per k-group for A and for B, pointing into the
+  // buffer being read; they flip between the two buffers once per slab. ----
+  const int h = lane >> 5;
+  const int sw = lane & 7;
+  int a_addr[4], b_addr[4];  // in f32x4 units
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    a_addr[g] = (wm * WM + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw);
+    b_addr[g] = BM * CHUNKS + (wn * WN + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw);
+  }
+  f32x4 af[2][TM], bf[2][TN];
+  auto read_ops = [&](int g, int p, int extra) {  // extra: 0 = current buffer, STAGE = other
+#pragma unroll
+    for (int i = 0; i < TM; i++) af[p][i] = lds[a_addr[g] + extra + i * 32 * CHUNKS];
+#pragma unroll
+    for (int j = 0; j < TN; j++) bf[p][j] = lds[b_addr[g] + extra + j * 32 * CHUNKS];
+  };
+  auto mfma_group = [&](int p) {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] =
+              __builtin_amdgcn_mfma_f32_32x32x2f32(af[p][i][e], bf[p][j][e], acc[i][j], 0, 0, 0);
+  };
+#define G2_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define G2_READS_IN_SHADOW()           \
+  _Pragma("unroll") for (int i_ = 0; i_ < TM + TN; i_++) { \
+    G2_SGB(0x008, 1);                  \
+    G2_SGB(0x100, 1);                  \
+  }
+
+  // Pipeline (two buffers; slab s lives in buffer s & 1):
+  //   groups 0..2 of slab s: MFMAs, each group reading the next group's operands
+  //   wait for this wave's DMAs of slab s+1, BARRIER: every wave's reads of slab s
+  //     are complete and every wave's DMAs of slab s+1 have landed
+  //   group 3: MFMAs, reading group 0 of slab s+1 and issuing the DMAs of slab s+2
+  //     into the buffer slab s just vacated
+  dma_slab(0, 0);
+  dma_slab(1, 1);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | DMA_PER);  // vmcnt(DMA_PER): slab 0 has landed
+  __syncthreads();
+  read_ops(0, 0, 0);
+  int flip = STAGE;  // offset from the buffer being read to the other one
+
+  for (int s = 0; s < nslab; s++) {
+    read_ops(1, 1, 0);
+    mfma_group(0);
+    read_ops(2, 0, 0);
+    mfma_group(1);
+    read_ops(3, 1, 0);
+    mfma_group(0);
+#pragma unroll
+    for (int g = 0; g < 3; g++) {
+      G2_READS_IN_SHADOW();
+      G2_SGB(0x008, MFMAS - (TM + TN));
+    }
+
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): my DMAs of slab s+1 have landed
+    __syncthreads();
+
+    read_ops(0, 0, flip);
+    dma_slab(s + 2, s & 1);
+    mfma_group(1);
+    G2_READS_IN_SHADOW();
+#pragma unroll
+    for (int i = 0; i < DMA_PER; i++) {
+      G2_SGB(0x008, 1);
+      G2_SGB(0x020, 1);
+    }
+    G2_SGB(0x008, MFMAS - (TM + TN) - DMA_PER);
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      a_addr[g] += flip;
+      b_addr[g] += flip;
+    }
+    flip = -flip;
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the (unused) DMAs before the LDS is released
+#undef G2_SGB
+#undef G2_READS_IN_SHADOW
+
+  // ---- epilogue -----------------------------------------------------------
+  const bool full = (m0 + BM <= M) && (n0 + BN <= N);
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int col = n0 + wn * WN + j * 32 + (lane & 31);
+      const int rbase = m0 + wm * WM + i * 32 + 4 * h;
+      float* o = out + (size_t)rbase * N + col;
+      if (full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          float r = acc[i][j][v];
+          if (GELU) r = gelu_tanh(r);
+          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
+        }
+      } else if (col < N) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int row = rbase + 8 * (v >> 2) + (v & 3);
+          if (row < M) {
+            float r = acc[i][j][v];
+            if (GELU) r = gelu_tanh(r);
+            out[(size_t)row * N + col] = r;
+          }
+        }
+      }
+    }
+  }
+}
+
 // Any shape, any alignment; one thread per output.  Only used when K is not a
 // multiple of 4 or an operand is not 16-byte aligned.
 __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const float* inp,
@@ -282,6 +484,26 @@ __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const f
   out[idx] = gelu ? gelu_tanh(acc) : acc;
 }
 
+// Sets the dynamic-LDS limit of a kernel once per (thread, device, kernel).
+template <typename F>
+static int allow_lds(F kfn, size_t lds_bytes, int slot) {
+  static thread_local int configured_for = -1;
+  static thread_local unsigned configured_mask = 0;
+  int dev = 0;
+  G2_HIP(hipGetDevice(&dev));
+  if (configured_for != dev) {
+    configured_for = dev;
+    configured_mask = 0;
+  }
+  if (!(configured_mask & (1u << slot))) {
+    G2_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    configured_mask |= 1u << slot;
+  }
+  return GPT2HIP_OK;
+}
+
+// Register-staged kernel: any K % 4 == 0.
 template <int BM, int BN, int WGM, int WGN>
 static int launch_mfma(float* out, const float* inp, const float* weight, const float* bias, int M,
                        int K, int N, bool gelu) {
@@ -295,20 +517,25 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
                            : matmul_mfma_kernel<BM, BN, WGM, WGN, false, true>)
                    : (gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true, false>
                            : matmul_mfma_kernel<BM, BN, WGM, WGN, false, false>);
-  static thread_local int configured_for = -1;  // device whose attribute was set (per variant)
-  static thread_local int configured_mask = 0;
-  int dev = 0;
-  G2_HIP(hipGetDevice(&dev));
-  if (configured_for != dev) {
-    configured_for = dev;
-    configured_mask = 0;
-  }
-  const int bit = (gelu ? 2 : 1) << (ktail ? 2 : 0);
-  if (!(configured_mask & bit)) {
-    G2_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    configured_mask |= bit;
-  }
+  if (int rc = allow_lds(kfn, lds_bytes, (gelu ? 1 : 0) + (ktail ? 2 : 0))) return rc;
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
+                     K, N, ntm, ntn);
+  G2_LAUNCH_CHECK("matmul_forward");
+  return GPT2HIP_OK;
+}
+
+// LDS-DMA kernel: K % 32 == 0.
+template <int BM, int BN, int WGM, int WGN, int SLOT>
+static int launch_dma(float* out, const float* inp, const float* weight, const float* bias, int M,
+                      int K, int N, bool gelu) {
+  constexpr int NT = WGM * WGN * kWave;
+  constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
+  const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
+  const long long tiles = (long long)ntm * ntn;
+  if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
+  auto kfn = gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true>
+                  : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
+  if (int rc = allow_lds(kfn, lds_bytes, SLOT + (gelu ? 1 : 0))) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
                      K, N, ntm, ntn);
   G2_LAUNCH_CHECK("matmul_forward");
@@ -330,6 +557,20 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
                        out, inp, weight, bias, M, C, OC, gelu ? 1 : 0);
     G2_LAUNCH_CHECK("matmul_forward");
     return GPT2HIP_OK;
+  }
+  // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
+  if (C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31)) {
+    // Tile choice by wave quantisation over the 256 CUs: time ~ rounds x tile area.
+    // 128x192 wins ties (fewer LDS reads per MFMA).
+    const long long t192 = (long long)((M + 127) / 128) * ((OC + 191) / 192);
+    const long long t128 = (long long)((M + 127) / 128) * ((OC + 127) / 128);
+    const long long cost192 = ((t192 + 255) / 256) * 3, cost128 = ((t128 + 255) / 256) * 2;
+    if (cost128 < cost192) return launch_dma<128, 128, 4, 2, 4>(out, inp, weight, bias, M, C, OC, gelu);
+    // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
+    // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
+    // gives every SIMD two waves to alternate between.
+    if (t192 >= 16 * 256) return launch_dma<128, 192, 2, 2, 0>(out, inp, weight, bias, M, C, OC, gelu);
+    return launch_dma<128, 192, 4, 2, 2>(out, inp, weight, bias, M, C, OC, gelu);
   }
   return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu);
 }
