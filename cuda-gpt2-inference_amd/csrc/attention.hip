@@ -5,16 +5,17 @@
 //
 // Shape of the computation (head size 64).  A workgroup of 4 waves owns 128
 // consecutive queries of one (batch, head); each wave owns 32 of them.  Keys
-// and values are staged through LDS in tiles of 64 keys (fetched into
-// registers one tile ahead, two LDS buffers, one barrier per tile); a wave
-// consumes a tile as two sub-tiles of 32 keys.
+// and values go from global memory straight into LDS (global_load_lds_dwordx4,
+// two buffers of 64 keys, one barrier per tile); a wave consumes a tile as two
+// sub-tiles of 32 keys.
 //
 // Per sub-tile a wave computes, with v_mfma_f32_32x32x2_f32,
 //     S^T (32 keys x 32 queries) = K_sub (32 x 64) . Q^T (64 x 32)
 // so that lane l owns query l%32 and holds 16 of that query's 32 scores
 // (keys 8*(v/4) + 4*(l/32) + v%4, v = 0..15); lane l^32 holds the other 16.
 // Row maxima and sums are therefore register reductions plus one exchange
-// with lane l^32.  The probabilities are then used IN PLACE as the B operand of
+// with lane l^32 (v_permlane32_swap).  The probabilities are then used IN PLACE
+// as the B operand of
 //     O^T (64 x 32 queries) += V_sub^T (64 x 32 keys) . P^T (32 keys x 32 queries)
 // because the accumulator layout of S^T is exactly a valid B-operand layout
 // once the k index of each MFMA is read as "key 8*(v/4)+v%4 for lanes 0..31,
@@ -28,6 +29,15 @@
 // accumulator a (0/1) of lane l, register v holds output feature
 // 16*(v/4) + 8*(l/32) + 2*(v%4) + a: eight consecutive floats per v/4, stored
 // as two 128-bit writes.
+//
+// Every VALU instruction takes issue time from the matrix pipe on this chip, so
+// the softmax is kept lean: hardware exp2 on a fused multiply-add, and a LAZY
+// running maximum — the shift m only moves when some score exceeds it by more
+// than 2^8 after scaling, so the rescaling of O and of the running sum is a rare,
+// wave-uniform branch.  Softmax is invariant to the shift, so this is exact;
+// probabilities are merely allowed to reach 2^8 instead of 1 before normalisation.
+// (The branch is taken per group of 32 queries, so the ROUNDING of a query's result
+// can depend on the other queries of its group; its value cannot.)
 #include "common.hpp"
 
 namespace g2 {
@@ -37,17 +47,45 @@ constexpr int BQ = 128;         // queries per workgroup (4 waves x 32)
 constexpr int BKV = 64;         // keys per LDS tile
 constexpr int KV_CH = HS / 4;   // 16-byte chunks per K/V row
 constexpr int ATT_THREADS = 256;
-constexpr int KV_PER = BKV * KV_CH / ATT_THREADS;  // chunks per thread per tensor = 4
+constexpr int ATT_WAVES = ATT_THREADS / kWave;
+constexpr int KV_TILE_BYTES = BKV * HS * 4;                 // 16 KiB per tensor per tile
+constexpr int KV_DMA_PER = 2 * (KV_TILE_BYTES / 1024) / ATT_WAVES;  // K+V DMAs per wave and tile = 8
+constexpr float LAZY_LOG2 = 8.0f;  // allowed growth of 2^x above the current shift
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void glb_void_t;
+
+// Exchange between lanes l and l^32: v_permlane32_swap swaps lanes 32..63 of its
+// first operand with lanes 0..31 of its second.  Fed two copies of x it leaves
+// {x[0..31], x[0..31]} in one and {x[32..63], x[32..63]} in the other, so either
+// reduction of the two registers is the l / l^32 pair reduction, in every lane.
+// Written as inline assembly so that both results are kept as distinct registers.
+__device__ __forceinline__ void pair_split(float x, float& lo, float& hi) {
+  lo = x;
+  hi = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float pair_max(float x) {
+  float lo, hi;
+  pair_split(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  float lo, hi;
+  pair_split(x, lo, hi);
+  return lo + hi;
+}
 
 __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
     float* __restrict__ out, const float* __restrict__ qkv, int T, int NH, int nqt,
     float scale_log2e) {
-  __shared__ f32x4 k_lds[2][BKV * KV_CH];
-  __shared__ f32x4 v_lds[2][BKV * KV_CH];
+  // [buffer][K tile | V tile]
+  __shared__ f32x4 kv_lds[2][2 * BKV * KV_CH];
+  char* const lds_bytes = reinterpret_cast<char*>(&kv_lds[0][0]);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h32 = lane >> 5;
   const int l32 = lane & 31;
 
@@ -61,8 +99,6 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
   const int C = NH * HS;
   const size_t row_stride = (size_t)3 * C;
   const float* base = qkv + (size_t)b * T * row_stride + head * HS;
-  const float* kbase = base + C;
-  const float* vbase = base + 2 * C;
 
   const int q0 = qtile * BQ;          // first query of the workgroup
   const int qw = q0 + wave * 32;      // first query of this wave
@@ -79,35 +115,32 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
     for (int g = 0; g < 8; g++) qreg[g] = qp[2 * g + h32];
   }
 
-  // ---- K/V staging ---------------------------------------------------------
-  f32x4 kst[KV_PER], vst[KV_PER];
-  int st_row[KV_PER], st_chunk[KV_PER];
+  // ---- K/V LDS-DMA: one instruction moves 4 rows of 256 bytes ------------------
+  // DMA j of this wave: group gi = wave*KV_DMA_PER + j of the tile's 32 groups
+  // (0..15: K rows 4*gi.., 16..31: V rows).  Lane l lands at LDS slot l of the group:
+  // row l/16, chunk position l%16; for K it fetches logical chunk (l%16) ^ (row & 7).
+  // Keys at or past T are clamped to T-1: they only ever meet queries < key, i.e. they
+  // are masked, or queries >= T, which are not stored.
+  const char* const kv_base = reinterpret_cast<const char*>(base + C);  // K; V is C floats on
+  int dma_row[KV_DMA_PER];       // row inside the tile
+  unsigned dma_col[KV_DMA_PER];  // byte offset inside the (K|V) row, V's includes +C floats
 #pragma unroll
-  for (int j = 0; j < KV_PER; j++) {
-    const int q = tid + j * ATT_THREADS;
-    st_row[j] = q >> 4;
-    st_chunk[j] = q & 15;
+  for (int j = 0; j < KV_DMA_PER; j++) {
+    const int gi = wave * KV_DMA_PER + j;
+    const bool is_v = gi >= 16;
+    const int row = 4 * (gi & 15) + (lane >> 4);
+    const int c = is_v ? (lane & 15) : ((lane & 15) ^ (row & 7));
+    dma_row[j] = row;
+    dma_col[j] = (unsigned)(c * 16 + (is_v ? C * 4 : 0));
   }
-  auto fetch = [&](int tile) {
+  auto dma_tile = [&](int tile, int buf) {
 #pragma unroll
-    for (int j = 0; j < KV_PER; j++) {
-      const int key = tile * BKV + st_row[j];
-      f32x4 kk = {0.f, 0.f, 0.f, 0.f}, vv = {0.f, 0.f, 0.f, 0.f};
-      if (key < kv_end) {
-        const size_t off = (size_t)key * row_stride + st_chunk[j] * 4;
-        kk = *reinterpret_cast<const f32x4*>(kbase + off);
-        vv = *reinterpret_cast<const f32x4*>(vbase + off);
-      }
-      kst[j] = kk;
-      vst[j] = vv;
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < KV_PER; j++) {
-      const int r = st_row[j], c = st_chunk[j];
-      k_lds[buf][r * KV_CH + (c ^ (r & 7))] = kst[j];
-      v_lds[buf][r * KV_CH + c] = vst[j];
+    for (int j = 0; j < KV_DMA_PER; j++) {
+      const int key = min(tile * BKV + dma_row[j], T - 1);
+      __builtin_amdgcn_global_load_lds(
+          (glb_void_t*)(kv_base + (size_t)key * (row_stride * 4) + dma_col[j]),
+          (lds_void_t*)(lds_bytes + buf * (2 * KV_TILE_BYTES) + (wave * KV_DMA_PER + j) * 1024),
+          16, 0, 0);
     }
   };
 
@@ -117,16 +150,21 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
     o0[v] = 0.f;
     o1[v] = 0.f;
   }
-  float m_run = -INFINITY;  // running max of raw (unscaled) scores of this lane's query
-  float l_run = 0.f;        // this lane's share of the running denominator
+  float m_used = -INFINITY;  // current shift, in raw (unscaled) score units
+  float mc = 0.f;            // m_used * scale_log2e (0 while m_used is -inf: see below)
+  float l_run = 0.f;         // this lane's share of the running denominator
+  const float lazy_raw = LAZY_LOG2 / scale_log2e;
 
-  fetch(0);
-  stash(0);
+  dma_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
 
   for (int tile = 0; tile < ntile; tile++) {
     const int buf = tile & 1;
-    if (tile + 1 < ntile) fetch(tile + 1);
+    // the other buffer was last read before the barrier that ended the previous tile
+    if (tile + 1 < ntile) dma_tile(tile + 1, buf ^ 1);
+    const f32x4* k_tile = &kv_lds[buf][0];
+    const f32x2* v_tile = reinterpret_cast<const f32x2*>(&kv_lds[buf][BKV * KV_CH]);
 
 #pragma unroll
     for (int sub = 0; sub < 2; sub++) {
@@ -137,7 +175,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
       f32x16 s;
 #pragma unroll
       for (int v = 0; v < 16; v++) s[v] = 0.f;
-      const f32x4* krow = &k_lds[buf][(sub * 32 + l32) * KV_CH];
+      const f32x4* krow = k_tile + (sub * 32 + l32) * KV_CH;
       const int sw = lane & 7;
 #pragma unroll
       for (int g = 0; g < 8; g++) {
@@ -156,45 +194,47 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
         }
       }
 
-      // online softmax for this lane's query
-      float mx = s[0];
+      // lazy online softmax for this lane's query
+      float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
 #pragma unroll
-      for (int v = 1; v < 16; v++) mx = fmaxf(mx, s[v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);  // finite: key k0 <= every query of the wave
-      const float alpha = exp2f((m_run - m_new) * scale_log2e);
-      m_run = m_new;
+      for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
+      mx = pair_max(fmaxf(mx, s[15]));  // finite: key k0 <= every query of the wave
+      if (__builtin_amdgcn_ballot_w64(mx > m_used + lazy_raw) != 0) {
+        const float m_new = fmaxf(m_used, mx);
+        const float alpha = __builtin_amdgcn_exp2f((m_used - m_new) * scale_log2e);  // 0 at first
+        m_used = m_new;
+        mc = m_new * scale_log2e;
+        l_run *= alpha;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          o0[v] *= alpha;
+          o1[v] *= alpha;
+        }
+      }
       float psum = 0.f;
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        s[v] = exp2f((s[v] - m_new) * scale_log2e);
+        s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], scale_log2e, -mc));
         psum += s[v];
       }
-      l_run = l_run * alpha + psum;
-#pragma unroll
-      for (int v = 0; v < 16; v++) {
-        o0[v] *= alpha;
-        o1[v] *= alpha;
-      }
+      l_run += psum;
 
       // O^T += V_sub^T . P^T
-      const f32x2* vrow = reinterpret_cast<const f32x2*>(&v_lds[buf][0]);
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int key = sub * 32 + 8 * (v >> 2) + 4 * h32 + (v & 3);
-        const f32x2 vv = vrow[key * (HS / 2) + l32];
+        const f32x2 vv = v_tile[key * (HS / 2) + l32];
         o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s[v], o0, 0, 0, 0);
         o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s[v], o1, 0, 0, 0);
       }
     }
 
-    if (tile + 1 < ntile) stash(buf ^ 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): my DMAs of the next tile have landed
     __syncthreads();
   }
 
   // ---- normalise and store -------------------------------------------------
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv = 1.0f / l_tot;
+  const float inv = 1.0f / pair_sum(l_run);
   if (myq < T) {
     float* op = out + ((size_t)b * T + myq) * C + head * HS + 8 * h32;
 #pragma unroll
