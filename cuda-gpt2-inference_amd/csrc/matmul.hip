@@ -24,6 +24,8 @@
 // a lane owns one output column, so the bias is folded into the accumulator's
 // initial value (as the reference does, 9_matmul_async_cg_tf32_gelu.cuh:56-84)
 // and every store instruction writes two 128-byte row segments.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace g2 {
@@ -312,34 +314,51 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   const int m0 = tm * BM, n0 = tn * BN;
 
   // ---- LDS-DMA descriptors -------------------------------------------------
-  // DMA j of this wave fills group gi = wave*DMA_PER + j (rows 8*gi .. 8*gi+7 of the
-  // buffer).  Rows past the end of a matrix are clamped to its last row: they only
-  // feed accumulator rows / columns that the epilogue does not store.
-  const char* dma_base[DMA_PER];  // wave-uniform: the tile's first row of A or of B
-  unsigned dma_off[DMA_PER];      // per lane: byte offset of its 16-byte chunk
+  // One DMA fills a group of 8 rows of a buffer.  Each wave owns A_PER groups of the A
+  // rows and B_PER groups of the B rows.  Rows past the end of a matrix are clamped to
+  // its last row: they only feed accumulator rows / columns that the epilogue does not
+  // store.  An address is a wave-uniform 64-bit base (the tile's first row of A or of
+  // B, moved on by one slab per iteration with scalar adds) plus a fixed 32-bit
+  // per-lane byte offset, so the loop spends no vector instructions on addressing.
+  constexpr int A_PER = BM / 8 / NW, B_PER = BN / 8 / NW;
+  static_assert(BM / 8 % NW == 0 && BN / 8 % NW == 0, "tile/waves mismatch");
+  const char* const a_tile = reinterpret_cast<const char*>(inp + (size_t)m0 * K);
+  const char* const b_tile = reinterpret_cast<const char*>(weight + (size_t)n0 * K);
+  unsigned dma_off[DMA_PER];
+  int dma_group[DMA_PER];  // wave-uniform: which 8-row group of the buffer
   {
     const int rr = lane >> 3, c = (lane & 7) ^ rr;
 #pragma unroll
     for (int j = 0; j < DMA_PER; j++) {
-      const int row = 8 * (wave * DMA_PER + j) + rr;
-      if (8 * (wave * DMA_PER + j) < BM) {
-        dma_base[j] = reinterpret_cast<const char*>(inp + (size_t)m0 * K);
+      if (j < A_PER) {
+        dma_group[j] = wave * A_PER + j;
+        const int row = 8 * dma_group[j] + rr;
         dma_off[j] = (unsigned)((min(m0 + row, M - 1) - m0) * K + c * 4) * 4u;
       } else {
-        dma_base[j] = reinterpret_cast<const char*>(weight + (size_t)n0 * K);
-        dma_off[j] = (unsigned)((min(n0 + row - BM, N - 1) - n0) * K + c * 4) * 4u;
+        dma_group[j] = BM / 8 + wave * B_PER + (j - A_PER);
+        const int row = 8 * (dma_group[j] - BM / 8) + rr;
+        dma_off[j] = (unsigned)((min(n0 + row, N - 1) - n0) * K + c * 4) * 4u;
       }
     }
   }
   const int nslab = K / BK;
   auto dma_slab = [&](int slab, int buf) {
     const size_t kbytes = (size_t)min(slab, nslab - 1) * (BK * 4);  // past the end: reload
+    const char* a_k = a_tile + kbytes;
+    const char* b_k = b_tile + kbytes;
+    // Opaque to the optimiser, so that "scalar base + 32-bit lane offset" reaches the
+    // instruction selector intact (it is the scalar-base addressing form of the load)
+    // instead of being re-associated into a 64-bit vector add per load.
+    asm volatile("" : "+s"(a_k), "+s"(b_k));
 #pragma unroll
     for (int j = 0; j < DMA_PER; j++)
       __builtin_amdgcn_global_load_lds(
-          (glb_void_t*)(dma_base[j] + kbytes + dma_off[j]),
-          (lds_void_t*)(lds_bytes + buf * STAGE_BYTES + (wave * DMA_PER + j) * 1024), 16, 0, 0);
+          (glb_void_t*)((j < A_PER ? a_k : b_k) + dma_off[j]),
+          (lds_void_t*)(lds_bytes + buf * STAGE_BYTES + dma_group[j] * 1024), 16, 0, 0);
   };
+  // the first two slabs are on their way before anything else is set up
+  dma_slab(0, 0);
+  dma_slab(1, 1);
 
   // ---- accumulators, initialised with the bias of the lane's column ----
   f32x16 acc[TM][TN];
@@ -353,22 +372,27 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
       for (int v = 0; v < 16; v++) acc[i][j][v] = bv;
   }
 
-  // ---- operand read addresses: one per k-group for A and for B, pointing into the
-  // buffer being read; they flip between the two buffers once per slab. ----
+  // ---- operand read addresses (bytes) inside buffer 0: one per k-group for A and
+  // for B.  The other buffer and the wave's further 32-row tiles are immediate
+  // offsets of the read instruction. ----
   const int h = lane >> 5;
   const int sw = lane & 7;
-  int a_addr[4], b_addr[4];  // in f32x4 units
+  int a_addr[4], b_addr[4];
 #pragma unroll
   for (int g = 0; g < 4; g++) {
-    a_addr[g] = (wm * WM + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw);
-    b_addr[g] = BM * CHUNKS + (wn * WN + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw);
+    a_addr[g] = ((wm * WM + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw)) * 16;
+    b_addr[g] = (BM * CHUNKS + (wn * WN + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw)) * 16;
   }
   f32x4 af[2][TM], bf[2][TN];
-  auto read_ops = [&](int g, int p, int extra) {  // extra: 0 = current buffer, STAGE = other
+  auto read_ops = [&](int g, int p, int buf) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) af[p][i] = lds[a_addr[g] + extra + i * 32 * CHUNKS];
+    for (int i = 0; i < TM; i++)
+      af[p][i] = *reinterpret_cast<const f32x4*>(lds_bytes + a_addr[g] +
+                                                 (buf * STAGE_BYTES + i * (32 * BK * 4)));
 #pragma unroll
-    for (int j = 0; j < TN; j++) bf[p][j] = lds[b_addr[g] + extra + j * 32 * CHUNKS];
+    for (int j = 0; j < TN; j++)
+      bf[p][j] = *reinterpret_cast<const f32x4*>(lds_bytes + b_addr[g] +
+                                                 (buf * STAGE_BYTES + j * (32 * BK * 4)));
   };
   auto mfma_group = [&](int p) {
 #pragma unroll
@@ -393,19 +417,14 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   //     are complete and every wave's DMAs of slab s+1 have landed
   //   group 3: MFMAs, reading group 0 of slab s+1 and issuing the DMAs of slab s+2
   //     into the buffer slab s just vacated
-  dma_slab(0, 0);
-  dma_slab(1, 1);
-  __builtin_amdgcn_s_waitcnt(0x0F70 | DMA_PER);  // vmcnt(DMA_PER): slab 0 has landed
-  __syncthreads();
-  read_ops(0, 0, 0);
-  int flip = STAGE;  // offset from the buffer being read to the other one
-
-  for (int s = 0; s < nslab; s++) {
-    read_ops(1, 1, 0);
+  // The slab loop is unrolled by two so that the buffer is a compile-time constant.
+  auto slab_body = [&](int s, auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+    read_ops(1, 1, buf);
     mfma_group(0);
-    read_ops(2, 0, 0);
+    read_ops(2, 0, buf);
     mfma_group(1);
-    read_ops(3, 1, 0);
+    read_ops(3, 1, buf);
     mfma_group(0);
 #pragma unroll
     for (int g = 0; g < 3; g++) {
@@ -416,8 +435,8 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): my DMAs of slab s+1 have landed
     __syncthreads();
 
-    read_ops(0, 0, flip);
-    dma_slab(s + 2, s & 1);
+    read_ops(0, 0, buf ^ 1);
+    dma_slab(s + 2, buf);
     mfma_group(1);
     G2_READS_IN_SHADOW();
 #pragma unroll
@@ -426,13 +445,16 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
       G2_SGB(0x020, 1);
     }
     G2_SGB(0x008, MFMAS - (TM + TN) - DMA_PER);
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      a_addr[g] += flip;
-      b_addr[g] += flip;
-    }
-    flip = -flip;
+  };
+  __builtin_amdgcn_s_waitcnt(0x0F70 | DMA_PER);  // vmcnt(DMA_PER): slab 0 has landed
+  __syncthreads();
+  read_ops(0, 0, 0);
+  int s = 0;
+  for (; s + 1 < nslab; s += 2) {
+    slab_body(s, std::integral_constant<int, 0>{});
+    slab_body(s + 1, std::integral_constant<int, 1>{});
   }
+  if (s < nslab) slab_body(s, std::integral_constant<int, 0>{});
   __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the (unused) DMAs before the LDS is released
 #undef G2_SGB
 #undef G2_READS_IN_SHADOW
