@@ -11,76 +11,91 @@
 
 namespace g2 {
 
-constexpr int kRowsPerBlock = 4;  // 4 waves = 256 threads
+constexpr int kWavesPerBlock = 4;  // 256 threads
 
-// NV float4 per lane cover C <= 256*NV.  FUSED adds inp2 and stores the sum.
-template <int NV, bool FUSED>
-__global__ __launch_bounds__(kRowsPerBlock* kWave) void layernorm_rows_kernel(
+// NV float4 per lane cover C <= 256*NV.  FUSED adds inp2 and stores the sum.  A wave
+// owns ROWS consecutive rows and issues all of their loads before it touches any of
+// them: at N = 8192 four rows per wave (a quarter of the waves, four times the bytes
+// in flight per wave) moved 72-76 % of HBM peak against 62-67 % for one row per wave.
+template <int NV, int ROWS, bool FUSED>
+__global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
     float* res_out, float* out, float* __restrict__ mean, float* __restrict__ rstd,
     const float* inp1, const float* inp2, const float* __restrict__ weight,
     const float* __restrict__ bias, int N, int C) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
-  if (row >= N) return;
+  const int row0 = (blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) * ROWS;
+  if (row0 >= N) return;
   const int C4 = C >> 2;
-  const size_t base = (size_t)row * C4;
-  const f32x4* x1 = reinterpret_cast<const f32x4*>(inp1) + base;
-  const f32x4* x2 = FUSED ? reinterpret_cast<const f32x4*>(inp2) + base : nullptr;
 
-  f32x4 v[NV];
+  f32x4 v[ROWS][NV];
 #pragma unroll
-  for (int j = 0; j < NV; j++) {
-    const int c = lane + j * kWave;
-    f32x4 a = {0.f, 0.f, 0.f, 0.f};
-    if (c < C4) {
-      a = __builtin_nontemporal_load(x1 + c);
-      if (FUSED) a += __builtin_nontemporal_load(x2 + c);
-    }
-    v[j] = a;
-  }
-  if (FUSED) {
-    f32x4* ro = reinterpret_cast<f32x4*>(res_out) + base;
+  for (int r = 0; r < ROWS; r++) {
+    const size_t base = (size_t)min(row0 + r, N - 1) * C4;  // rows past N: reloaded, never stored
+    const f32x4* x1 = reinterpret_cast<const f32x4*>(inp1) + base;
+    const f32x4* x2 = FUSED ? reinterpret_cast<const f32x4*>(inp2) + base : nullptr;
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int c = lane + j * kWave;
-      if (c < C4) ro[c] = v[j];
+      f32x4 a = {0.f, 0.f, 0.f, 0.f};
+      if (c < C4) {
+        a = __builtin_nontemporal_load(x1 + c);
+        if (FUSED) a += __builtin_nontemporal_load(x2 + c);
+      }
+      v[r][j] = a;
     }
-  }
-
-  float s = 0.f;
-#pragma unroll
-  for (int j = 0; j < NV; j++) s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
-  const float m = wave_sum(s) / (float)C;
-
-  float q = 0.f;
-#pragma unroll
-  for (int j = 0; j < NV; j++) {
-    const int c = lane + j * kWave;
-    if (c < C4) {
-      const f32x4 d = v[j] - m;
-      q += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
-    }
-  }
-  const float var = wave_sum(q) / (float)C;
-  const float rs = 1.0f / sqrtf(var + 1e-5f);
-
-  if (lane == 0) {
-    if (mean) mean[row] = m;
-    if (rstd) rstd[row] = rs;
   }
 
   const f32x4* w4 = reinterpret_cast<const f32x4*>(weight);
   const f32x4* b4 = reinterpret_cast<const f32x4*>(bias);
-  f32x4* o = reinterpret_cast<f32x4*>(out) + base;
 #pragma unroll
-  for (int j = 0; j < NV; j++) {
-    const int c = lane + j * kWave;
-    if (c < C4) {
-      const f32x4 n = (v[j] - m) * rs;
-      o[c] = n * w4[c] + b4[c];
+  for (int r = 0; r < ROWS; r++) {
+    const int row = row0 + r;
+    if (row >= N) break;
+    const size_t base = (size_t)row * C4;
+    if (FUSED) {
+      f32x4* ro = reinterpret_cast<f32x4*>(res_out) + base;
+#pragma unroll
+      for (int j = 0; j < NV; j++) {
+        const int c = lane + j * kWave;
+        if (c < C4) ro[c] = v[r][j];
+      }
+    }
+
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) s += (v[r][j].x + v[r][j].y) + (v[r][j].z + v[r][j].w);
+    const float m = wave_sum(s) / (float)C;
+
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int c = lane + j * kWave;
+      if (c < C4) {
+        const f32x4 d = v[r][j] - m;
+        q += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
+      }
+    }
+    const float var = wave_sum(q) / (float)C;
+    const float rs = 1.0f / sqrtf(var + 1e-5f);
+
+    if (lane == 0) {
+      if (mean) mean[row] = m;
+      if (rstd) rstd[row] = rs;
+    }
+
+    f32x4* o = reinterpret_cast<f32x4*>(out) + base;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      const int c = lane + j * kWave;
+      if (c < C4) {
+        const f32x4 n = (v[r][j] - m) * rs;
+        o[c] = n * w4[c] + b4[c];
+      }
     }
   }
 }
+
+constexpr int kRowsPerBlock = kWavesPerBlock;  // generic kernel: one row per wave
 
 // Any C, any alignment: one wave per row, three passes over global memory.
 template <bool FUSED>
@@ -130,29 +145,40 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   if (N == 0) return GPT2HIP_OK;
   if (!out || !inp1 || !weight || !bias || (FUSED && (!res_out || !inp2)))
     return fail(GPT2HIP_EINVAL, "%s: null pointer", name);
-  const dim3 grid((N + kRowsPerBlock - 1) / kRowsPerBlock), block(kRowsPerBlock * kWave);
+  const dim3 block(kWavesPerBlock * kWave);
   const bool vec = (C % 4 == 0) && C <= 4096 && aligned16(out) && aligned16(inp1) &&
                    aligned16(weight) && aligned16(bias) &&
                    (!FUSED || (aligned16(res_out) && aligned16(inp2)));
-#define G2_LN(NV)                                                                              \
-  hipLaunchKernelGGL((layernorm_rows_kernel<NV, FUSED>), grid, block, 0, 0, res_out, out, mean, \
-                     rstd, inp1, inp2, weight, bias, N, C)
+  // four rows per wave once there are enough rows to still fill the chip
+  const bool wide = N >= 4096;
+#define G2_LN(NV, ROWS)                                                                         \
+  hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED>),                                  \
+                     dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, 0, \
+                     res_out, out, mean, rstd, inp1, inp2, weight, bias, N, C)
+#define G2_LN_ROWS(NV) \
+  if (wide) {          \
+    G2_LN(NV, 4);      \
+  } else {             \
+    G2_LN(NV, 1);      \
+  }
   if (!vec) {
-    hipLaunchKernelGGL((layernorm_rows_generic_kernel<FUSED>), grid, block, 0, 0, res_out, out,
+    hipLaunchKernelGGL((layernorm_rows_generic_kernel<FUSED>),
+                       dim3((N + kRowsPerBlock - 1) / kRowsPerBlock), block, 0, 0, res_out, out,
                        mean, rstd, inp1, inp2, weight, bias, N, C);
   } else if (C <= 256) {
-    G2_LN(1);
+    G2_LN_ROWS(1)
   } else if (C <= 512) {
-    G2_LN(2);
+    G2_LN_ROWS(2)
   } else if (C <= 768) {
-    G2_LN(3);
+    G2_LN_ROWS(3)
   } else if (C <= 1024) {
-    G2_LN(4);
+    G2_LN_ROWS(4)
   } else if (C <= 2048) {
-    G2_LN(8);
+    G2_LN_ROWS(8)
   } else {
-    G2_LN(16);
+    G2_LN(16, 1);
   }
+#undef G2_LN_ROWS
 #undef G2_LN
   G2_LAUNCH_CHECK(name);
   return GPT2HIP_OK;
