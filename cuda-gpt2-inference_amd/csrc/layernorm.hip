@@ -17,7 +17,9 @@ constexpr int kWavesPerBlock = 4;  // 256 threads
 // owns ROWS consecutive rows and issues all of their loads before it touches any of
 // them: at N = 8192 four rows per wave (a quarter of the waves, four times the bytes
 // in flight per wave) moved 72-76 % of HBM peak against 62-67 % for one row per wave.
-template <int NV, int ROWS, bool FUSED>
+// EXACT (C == 256*NV and N % ROWS == 0, true for GPT-2) removes every bounds check, so
+// that the loads are issued as one unconditional batch.
+template <int NV, int ROWS, bool FUSED, bool EXACT>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
     float* res_out, float* out, float* __restrict__ mean, float* __restrict__ rstd,
     const float* inp1, const float* inp2, const float* __restrict__ weight,
@@ -30,14 +32,15 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
   f32x4 v[ROWS][NV];
 #pragma unroll
   for (int r = 0; r < ROWS; r++) {
-    const size_t base = (size_t)min(row0 + r, N - 1) * C4;  // rows past N: reloaded, never stored
+    // rows past N: reloaded, never stored
+    const size_t base = (size_t)(EXACT ? row0 + r : min(row0 + r, N - 1)) * C4;
     const f32x4* x1 = reinterpret_cast<const f32x4*>(inp1) + base;
     const f32x4* x2 = FUSED ? reinterpret_cast<const f32x4*>(inp2) + base : nullptr;
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int c = lane + j * kWave;
       f32x4 a = {0.f, 0.f, 0.f, 0.f};
-      if (c < C4) {
+      if (EXACT || c < C4) {
         a = __builtin_nontemporal_load(x1 + c);
         if (FUSED) a += __builtin_nontemporal_load(x2 + c);
       }
@@ -50,14 +53,14 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
 #pragma unroll
   for (int r = 0; r < ROWS; r++) {
     const int row = row0 + r;
-    if (row >= N) break;
+    if (!EXACT && row >= N) break;
     const size_t base = (size_t)row * C4;
     if (FUSED) {
       f32x4* ro = reinterpret_cast<f32x4*>(res_out) + base;
 #pragma unroll
       for (int j = 0; j < NV; j++) {
         const int c = lane + j * kWave;
-        if (c < C4) ro[c] = v[r][j];
+        if (EXACT || c < C4) ro[c] = v[r][j];
       }
     }
 
@@ -70,7 +73,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int c = lane + j * kWave;
-      if (c < C4) {
+      if (EXACT || c < C4) {
         const f32x4 d = v[r][j] - m;
         q += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
       }
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int c = lane + j * kWave;
-      if (c < C4) {
+      if (EXACT || c < C4) {
         const f32x4 n = (v[r][j] - m) * rs;
         o[c] = n * w4[c] + b4[c];
       }
@@ -151,15 +154,17 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
                    (!FUSED || (aligned16(res_out) && aligned16(inp2)));
   // four rows per wave once there are enough rows to still fill the chip
   const bool wide = N >= 4096;
-#define G2_LN(NV, ROWS)                                                                         \
-  hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED>),                                  \
+#define G2_LN(NV, ROWS, EXACT)                                                                  \
+  hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED, EXACT>),                           \
                      dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, 0, \
                      res_out, out, mean, rstd, inp1, inp2, weight, bias, N, C)
-#define G2_LN_ROWS(NV) \
-  if (wide) {          \
-    G2_LN(NV, 4);      \
-  } else {             \
-    G2_LN(NV, 1);      \
+#define G2_LN_ROWS(NV)                         \
+  if (wide && C == 256 * NV && N % 4 == 0) {   \
+    G2_LN(NV, 4, true);                        \
+  } else if (wide) {                           \
+    G2_LN(NV, 4, false);                       \
+  } else {                                     \
+    G2_LN(NV, 1, false);                       \
   }
   if (!vec) {
     hipLaunchKernelGGL((layernorm_rows_generic_kernel<FUSED>),
@@ -176,7 +181,7 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   } else if (C <= 2048) {
     G2_LN_ROWS(8)
   } else {
-    G2_LN(16, 1);
+    G2_LN(16, 1, false);
   }
 #undef G2_LN_ROWS
 #undef G2_LN
