@@ -27,6 +27,12 @@ if ROOT not in sys.path:
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
+# HBM bytes per launch of the dominant GEMM kernel (mean of the qkv, attproj and fcproj
+# shapes at M = 8192), from two `rocprofv3 --pmc` runs of `bench.py --pmc-probe`:
+# FETCH_SIZE (scaled x2.0: a 256 MiB copy reads 131 084 KiB on that counter) and
+# WRITE_SIZE (scale 1.0: the same copy writes 262 144 KiB).
+DOMINANT_TRAFFIC_BYTES = int((60816.6 + 21564.8 + 86076.5) / 3 * 2.0 * 1024
+                             + (73728 + 24576 + 24576) / 3 * 1024)
 
 
 def log(*a):
@@ -180,6 +186,40 @@ def standalone(g2):
     return out
 
 
+def pmc_probe(g2):
+    """One launch of every kernel at its BASELINE shape plus a plain copy of known size,
+    for `rocprofv3 --pmc` runs: the copy calibrates FETCH_SIZE / WRITE_SIZE."""
+    import torch
+    dev = "cuda"
+    M = 8192
+    src = torch.randn(64 << 20, device=dev)          # 256 MiB
+    dst = torch.empty_like(src)
+    for _ in range(2):
+        dst.copy_(src)                                # plain copy: reads 256 MiB, writes 256 MiB
+    for (C, OC) in ((768, 2304), (768, 768), (768, 3072), (3072, 768), (768, 50257)):
+        x = torch.randn(M, C, device=dev)
+        w = torch.randn(OC, C, device=dev) * 0.02
+        o = torch.empty(M, OC, device=dev)
+        for _ in range(2):
+            g2.matmul_forward(o, x, w, None, 8, 1024, C, OC)
+        del x, w, o
+    for C in (768, 1024):
+        x = torch.randn(M, C, device=dev)
+        r = torch.randn(M, C, device=dev)
+        o = torch.empty(M, C, device=dev)
+        s2 = torch.empty(M, C, device=dev)
+        w = torch.ones(C, device=dev)
+        b = torch.zeros(C, device=dev)
+        dst.copy_(src)                                # push the operands out of the caches
+        g2.fused_residual_layernorm_forward(s2, o, None, None, x, r, w, b, 8, 1024, C)
+    qkv = torch.randn(8, 1024, 3 * 768, device=dev)
+    o = torch.empty(8, 1024, 768, device=dev)
+    for _ in range(2):
+        g2.attention_forward(o, None, None, qkv, 8, 1024, 768, 12)
+    torch.cuda.synchronize()
+    print(json.dumps({"pmc_probe": "done", "copy_bytes_each_way": src.numel() * 4}))
+
+
 def cpu_baseline(model, cfg, B, T):
     """The CPU oracle on the host cores: one forward of the whole benchmark batch
     (a few seconds on 16 cores), after one untimed pass at B=1 to warm the threads."""
@@ -207,6 +247,8 @@ def main():
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--no-standalone", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="launch each kernel once plus a calibration copy (for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (the forward pass shards over the batch with "
@@ -222,6 +264,9 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
 
+    if args.pmc_probe:
+        pmc_probe(g2)
+        return
     cfg = dict(g2.GPT2_124M if args.model == "124M" else g2.GPT2_350M)
     B = args.batch or (8 if args.model == "124M" else 4)
     T = 1024
@@ -269,15 +314,18 @@ def main():
         kernels.append(row)
         log(f"  {k:26s} {prof[k]:8.3f} ms/fwd  " + (f"{row.get('TFLOP/s', 0):7.1f} TFLOP/s"
             if k in flops else f"{row.get('GB/s', 0):7.0f} GB/s"))
-    # dominant kernel: the bias (non-GELU) instantiation of the MFMA GEMM
-    dom = ("matmul_qkv", "matmul_attproj", "matmul_fcproj", "matmul_lmhead")
-    dom_launches = 3 * L + 1
+    # Dominant kernel symbol: matmul_dma_kernel<128,192,4,2,false>, the instantiation that
+    # runs the qkv, attention-projection and fc-projection GEMMs (3 per layer; the fc GEMM
+    # with its GELU epilogue and the lm-head are other instantiations of the same source).
+    dom = ("matmul_qkv", "matmul_attproj", "matmul_fcproj")
+    dom_launches = 3 * L
     dom_flops = sum(flops[k] for k in dom) / dom_launches
     dom_ms = sum(prof[k] for k in dom) / dom_launches
     achieved = dom_flops / dom_ms / 1e9
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
-                "kernel": "matmul_mfma_kernel<128,192,4,2,false>",
+                "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+                "traffic": DOMINANT_TRAFFIC_BYTES if (args.model == "124M" and B == 8) else None,
+                "kernel": "matmul_dma_kernel<128,192,4,2,false>",
                 "avg_launch_ms": dom_ms, "flops_per_launch": dom_flops,
                 "launches_per_forward": dom_launches}
 
