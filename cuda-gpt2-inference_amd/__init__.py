@@ -25,6 +25,9 @@ HIPCC_FLAGS = (
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
     # packed-fp32 VALU forms are switched off for every HIP translation unit
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # keep MFMA accumulators in ordinary VGPRs: the softmax reads them with VALU
+    # instructions, and copies out of the accumulation registers would cost issue slots
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 )
 
 EXPORTS = (

@@ -3,11 +3,18 @@
 // reference 3_flash_attention_permute.cuh:346-355 — as one flash-style kernel
 // on the fp32 matrix cores.  The T x T scores never leave registers.
 //
-// Shape of the computation (head size 64).  A workgroup of 4 waves owns 128
-// consecutive queries of one (batch, head); each wave owns 32 of them.  Keys
-// and values go from global memory straight into LDS (global_load_lds_dwordx4,
-// two buffers of 64 keys, one barrier per tile); a wave consumes a tile as two
-// sub-tiles of 32 keys.
+// Shape of the computation (head size 64).  A workgroup of 4 waves owns 64
+// consecutive queries of one (batch, head): two groups of 32 queries, each shared
+// by a PAIR of waves that split the keys between them.  Keys and values go from
+// global memory straight into LDS (global_load_lds_dwordx4, two buffers of 64
+// keys, one barrier per tile); of every tile the first wave of a pair takes the
+// first 32 keys and the second wave the last 32, each with its own running
+// maximum, sum and output, and the two partial results are merged once at the
+// end.  Splitting keys rather than queries keeps the four waves of a workgroup
+// equally busy under the causal mask (they differ by at most one sub-tile, on the
+// diagonal), which a split by queries does not: with 128 queries per workgroup and
+// one group per wave, non-causal attention ran at 80 % of the matrix peak and
+// causal attention at 60 %.
 //
 // Per sub-tile a wave computes, with v_mfma_f32_32x32x2_f32,
 //     S^T (32 keys x 32 queries) = K_sub (32 x 64) . Q^T (64 x 32)
@@ -38,12 +45,14 @@
 // probabilities are merely allowed to reach 2^8 instead of 1 before normalisation.
 // (The branch is taken per group of 32 queries, so the ROUNDING of a query's result
 // can depend on the other queries of its group; its value cannot.)
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace g2 {
 
 constexpr int HS = 64;          // head size this kernel is built for
-constexpr int BQ = 128;         // queries per workgroup (4 waves x 32)
+constexpr int BQ = 64;          // queries per workgroup (2 groups of 32, 2 waves each)
 constexpr int BKV = 64;         // keys per LDS tile
 constexpr int KV_CH = HS / 4;   // 16-byte chunks per K/V row
 constexpr int ATT_THREADS = 256;
@@ -101,7 +110,9 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
   const float* base = qkv + (size_t)b * T * row_stride + head * HS;
 
   const int q0 = qtile * BQ;          // first query of the workgroup
-  const int qw = q0 + wave * 32;      // first query of this wave
+  const int qgroup = wave >> 1;       // which 32 queries
+  const int khalf = wave & 1;         // which 32 keys of every 64-key tile
+  const int qw = q0 + qgroup * 32;    // first query of this wave
   const int myq = qw + l32;           // this lane's query
   const int kv_end = min(T, q0 + BQ); // keys the workgroup needs: [0, kv_end)
   const int ntile = (kv_end + BKV - 1) / BKV;
@@ -119,11 +130,15 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
   // DMA j of this wave: group gi = wave*KV_DMA_PER + j of the tile's 32 groups
   // (0..15: K rows 4*gi.., 16..31: V rows).  Lane l lands at LDS slot l of the group:
   // row l/16, chunk position l%16; for K it fetches logical chunk (l%16) ^ (row & 7).
-  // Keys at or past T are clamped to T-1: they only ever meet queries < key, i.e. they
-  // are masked, or queries >= T, which are not stored.
+  // An address is a wave-uniform base (the tile's first K row, moved on with scalar
+  // adds) plus a fixed 32-bit per-lane offset.  Only a last, partial tile (T % 64 != 0)
+  // needs per-lane work: keys at or past T are clamped to T-1 there; they only ever
+  // meet queries < key, i.e. they are masked, or queries >= T, which are not stored.
   const char* const kv_base = reinterpret_cast<const char*>(base + C);  // K; V is C floats on
+  const unsigned row_bytes = (unsigned)(row_stride * 4);
   int dma_row[KV_DMA_PER];       // row inside the tile
   unsigned dma_col[KV_DMA_PER];  // byte offset inside the (K|V) row, V's includes +C floats
+  unsigned dma_off[KV_DMA_PER];  // dma_row * row_bytes + dma_col
 #pragma unroll
   for (int j = 0; j < KV_DMA_PER; j++) {
     const int gi = wave * KV_DMA_PER + j;
@@ -132,15 +147,25 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
     const int c = is_v ? (lane & 15) : ((lane & 15) ^ (row & 7));
     dma_row[j] = row;
     dma_col[j] = (unsigned)(c * 16 + (is_v ? C * 4 : 0));
+    dma_off[j] = (unsigned)row * row_bytes + dma_col[j];
   }
   auto dma_tile = [&](int tile, int buf) {
+    const char* tile_base = kv_base + (size_t)tile * BKV * row_bytes;
+    char* const dst = lds_bytes + buf * (2 * KV_TILE_BYTES) + wave * (KV_DMA_PER * 1024);
+    if ((tile + 1) * BKV <= T) {
+      asm volatile("" : "+s"(tile_base));  // keep "scalar base + lane offset" intact for selection
 #pragma unroll
-    for (int j = 0; j < KV_DMA_PER; j++) {
-      const int key = min(tile * BKV + dma_row[j], T - 1);
-      __builtin_amdgcn_global_load_lds(
-          (glb_void_t*)(kv_base + (size_t)key * (row_stride * 4) + dma_col[j]),
-          (lds_void_t*)(lds_bytes + buf * (2 * KV_TILE_BYTES) + (wave * KV_DMA_PER + j) * 1024),
-          16, 0, 0);
+      for (int j = 0; j < KV_DMA_PER; j++)
+        __builtin_amdgcn_global_load_lds((glb_void_t*)(tile_base + dma_off[j]),
+                                         (lds_void_t*)(dst + j * 1024), 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < KV_DMA_PER; j++) {
+        const int key = min(tile * BKV + dma_row[j], T - 1);
+        __builtin_amdgcn_global_load_lds(
+            (glb_void_t*)(kv_base + (size_t)key * row_bytes + dma_col[j]),
+            (lds_void_t*)(dst + j * 1024), 16, 0, 0);
+      }
     }
   };
 
@@ -151,98 +176,160 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
     o1[v] = 0.f;
   }
   float m_used = -INFINITY;  // current shift, in raw (unscaled) score units
-  float mc = 0.f;            // m_used * scale_log2e (0 while m_used is -inf: see below)
+  float mc = 0.f;            // m_used * scale_log2e (unused while m_used is -inf)
   float l_run = 0.f;         // this lane's share of the running denominator
   const float lazy_raw = LAZY_LOG2 / scale_log2e;
 
-  dma_tile(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  __syncthreads();
+  // LDS read addresses (bytes, inside buffer 0, sub-tile 0); buffer and sub-tile are
+  // immediate offsets of the read instructions.
+  int k_addr[8];
+#pragma unroll
+  for (int g = 0; g < 8; g++) k_addr[g] = (l32 * KV_CH + ((2 * g + h32) ^ (lane & 7))) * 16;
+  const int v_addr = KV_TILE_BYTES + (4 * h32) * (HS * 4) + l32 * 8;
 
-  for (int tile = 0; tile < ntile; tile++) {
-    const int buf = tile & 1;
+  // Operand registers of one sub-tile: K as eight 16-byte chunks (A operand of the
+  // score MFMAs), V as sixteen 8-byte pairs (A operand of the output MFMAs).
+  struct Operands {
+    f32x4 k[8];
+    f32x2 v[16];
+  };
+  // All LDS reads of a sub-tile are issued in one batch, well before their first use:
+  // V is read before the score MFMAs that precede its use, and the next sub-tile's K
+  // before the output MFMAs of the current one.
+  auto read_k = [&](Operands& op, int off) {
+#pragma unroll
+    for (int g = 0; g < 8; g++)
+      op.k[g] = *reinterpret_cast<const f32x4*>(lds_bytes + k_addr[g] + off);
+  };
+  auto read_v = [&](Operands& op, int off) {
+#pragma unroll
+    for (int v = 0; v < 16; v++)
+      op.v[v] = *reinterpret_cast<const f32x2*>(lds_bytes + v_addr +
+                                                (off + (8 * (v >> 2) + (v & 3)) * (HS * 4)));
+  };
+
+  // Scores, lazy online softmax and output update of one sub-tile of 32 keys.
+  auto sub_tile = [&](int k0, const Operands& op, auto&& before_output) {
+    // S^T = K_sub . Q^T
+    f32x16 s;
+#pragma unroll
+    for (int v = 0; v < 16; v++) s[v] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; g++)
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(op.k[g][e], qreg[g][e], s, 0, 0, 0);
+
+    // causal mask on the diagonal sub-tile
+    if (k0 + 31 > qw) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int key = k0 + 8 * (v >> 2) + 4 * h32 + (v & 3);
+        if (key > myq) s[v] = -INFINITY;
+      }
+    }
+
+    // lazy online softmax for this lane's query
+    float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+    for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
+    mx = pair_max(fmaxf(mx, s[15]));  // finite: key k0 <= every query of the wave
+    if (__builtin_amdgcn_ballot_w64(mx > m_used + lazy_raw) != 0) {
+      const float m_new = fmaxf(m_used, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_used - m_new) * scale_log2e);  // 0 at first
+      m_used = m_new;
+      mc = m_new * scale_log2e;
+      l_run *= alpha;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        o0[v] *= alpha;
+        o1[v] *= alpha;
+      }
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], scale_log2e, -mc));
+      psum += s[v];
+    }
+    l_run += psum;
+
+    before_output();
+
+    // O^T += V_sub^T . P^T : register v pairs with key 8*(v/4) + 4*h32 + v%4
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(op.v[v].x, s[v], o0, 0, 0, 0);
+      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(op.v[v].y, s[v], o1, 0, 0, 0);
+    }
+  };
+
+  // One tile of 64 keys out of buffer BUF (a compile-time constant, so that every LDS
+  // address is register + immediate).
+  auto tile_body = [&](int tile, auto buf_tag) {
+    constexpr int BUF = decltype(buf_tag)::value;
+    constexpr int kbuf = BUF * (2 * KV_TILE_BYTES);
+    constexpr int sub1 = 32 * (HS * 4);
     // the other buffer was last read before the barrier that ended the previous tile
-    if (tile + 1 < ntile) dma_tile(tile + 1, buf ^ 1);
-    const f32x4* k_tile = &kv_lds[buf][0];
-    const f32x2* v_tile = reinterpret_cast<const f32x2*>(&kv_lds[buf][BKV * KV_CH]);
+    if (tile + 1 < ntile) dma_tile(tile + 1, BUF ^ 1);
 
-#pragma unroll
-    for (int sub = 0; sub < 2; sub++) {
-      const int k0 = tile * BKV + sub * 32;  // first key of the sub-tile
-      if (k0 > qw + 31 || k0 >= T) continue; // wave-uniform: nothing at or below the diagonal
-
-      // S^T = K_sub . Q^T
-      f32x16 s;
-#pragma unroll
-      for (int v = 0; v < 16; v++) s[v] = 0.f;
-      const f32x4* krow = k_tile + (sub * 32 + l32) * KV_CH;
-      const int sw = lane & 7;
-#pragma unroll
-      for (int g = 0; g < 8; g++) {
-        const f32x4 kk = krow[(2 * g + h32) ^ sw];
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-          s = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[e], qreg[g][e], s, 0, 0, 0);
-      }
-
-      // causal mask on the diagonal sub-tile
-      if (k0 + 31 > qw) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const int key = k0 + 8 * (v >> 2) + 4 * h32 + (v & 3);
-          if (key > myq) s[v] = -INFINITY;
-        }
-      }
-
-      // lazy online softmax for this lane's query
-      float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
-#pragma unroll
-      for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
-      mx = pair_max(fmaxf(mx, s[15]));  // finite: key k0 <= every query of the wave
-      if (__builtin_amdgcn_ballot_w64(mx > m_used + lazy_raw) != 0) {
-        const float m_new = fmaxf(m_used, mx);
-        const float alpha = __builtin_amdgcn_exp2f((m_used - m_new) * scale_log2e);  // 0 at first
-        m_used = m_new;
-        mc = m_new * scale_log2e;
-        l_run *= alpha;
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          o0[v] *= alpha;
-          o1[v] *= alpha;
-        }
-      }
-      float psum = 0.f;
-#pragma unroll
-      for (int v = 0; v < 16; v++) {
-        s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], scale_log2e, -mc));
-        psum += s[v];
-      }
-      l_run += psum;
-
-      // O^T += V_sub^T . P^T
-#pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const int key = sub * 32 + 8 * (v >> 2) + 4 * h32 + (v & 3);
-        const f32x2 vv = v_tile[key * (HS / 2) + l32];
-        o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s[v], o0, 0, 0, 0);
-        o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s[v], o1, 0, 0, 0);
-      }
+    // this wave's 32 keys of the tile; wave-uniform: do they reach down to the diagonal?
+    const int k0 = tile * BKV + khalf * 32;
+    if (k0 <= qw + 31 && k0 < T) {
+      Operands a;
+      read_k(a, kbuf + khalf * sub1);
+      read_v(a, kbuf + khalf * sub1);
+      sub_tile(k0, a, []() {});
     }
 
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): my DMAs of the next tile have landed
     __syncthreads();
-  }
+  };
 
-  // ---- normalise and store -------------------------------------------------
-  const float inv = 1.0f / pair_sum(l_run);
-  if (myq < T) {
-    float* op = out + ((size_t)b * T + myq) * C + head * HS + 8 * h32;
+  dma_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  int tile = 0;
+  for (; tile + 1 < ntile; tile += 2) {
+    tile_body(tile, std::integral_constant<int, 0>{});
+    tile_body(tile + 1, std::integral_constant<int, 1>{});
+  }
+  if (tile < ntile) tile_body(tile, std::integral_constant<int, 0>{});
+
+  // ---- merge the two key halves of each query group --------------------------
+  // The K/V buffers are idle after the loop's last barrier; the second wave of each
+  // pair parks its partial state there, one float per (register, lane).
+  float* const park = reinterpret_cast<float*>(lds_bytes) + qgroup * (35 * kWave) + lane;
+  if (khalf == 1) {
 #pragma unroll
-    for (int q4 = 0; q4 < 4; q4++) {
-      f32x4 lo = {o0[4 * q4 + 0], o1[4 * q4 + 0], o0[4 * q4 + 1], o1[4 * q4 + 1]};
-      f32x4 hi = {o0[4 * q4 + 2], o1[4 * q4 + 2], o0[4 * q4 + 3], o1[4 * q4 + 3]};
-      *reinterpret_cast<f32x4*>(op + 16 * q4) = lo * inv;
-      *reinterpret_cast<f32x4*>(op + 16 * q4 + 4) = hi * inv;
+    for (int v = 0; v < 16; v++) {
+      park[v * kWave] = o0[v];
+      park[(16 + v) * kWave] = o1[v];
+    }
+    park[32 * kWave] = m_used;
+    park[33 * kWave] = l_run;
+  }
+  __syncthreads();
+  if (khalf == 0) {
+    const float m1 = park[32 * kWave], l1 = park[33 * kWave];
+    const float m = fmaxf(m_used, m1);  // m_used is finite: key 0 is visible to every query
+    const float a0 = __builtin_amdgcn_exp2f((m_used - m) * scale_log2e);
+    const float a1 = __builtin_amdgcn_exp2f((m1 - m) * scale_log2e);  // 0 if that half saw no key
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      o0[v] = o0[v] * a0 + park[v * kWave] * a1;
+      o1[v] = o1[v] * a0 + park[(16 + v) * kWave] * a1;
+    }
+    const float inv = 1.0f / pair_sum(l_run * a0 + l1 * a1);
+    if (myq < T) {
+      float* op = out + ((size_t)b * T + myq) * C + head * HS + 8 * h32;
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        f32x4 lo = {o0[4 * q4 + 0], o1[4 * q4 + 0], o0[4 * q4 + 1], o1[4 * q4 + 1]};
+        f32x4 hi = {o0[4 * q4 + 2], o1[4 * q4 + 2], o0[4 * q4 + 3], o1[4 * q4 + 3]};
+        *reinterpret_cast<f32x4*>(op + 16 * q4) = lo * inv;
+        *reinterpret_cast<f32x4*>(op + 16 * q4 + 4) = hi * inv;
+      }
     }
   }
 }
