@@ -41,6 +41,7 @@ EXPORTS = (
     "matmul_forward_gelu", "matmul_forward_gelu_status",
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
+    "gpt2_checkpoint_read_config", "gpt2_build_from_checkpoint",
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
     "gpt2_forward_device_status", "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
@@ -109,6 +110,10 @@ def lib() -> ctypes.CDLL:
             f.argtypes, f.restype = args, ci
         L.gpt2_create.argtypes, L.gpt2_create.restype = [ctypes.POINTER(GPT2Config)], vp
         L.gpt2_destroy.argtypes, L.gpt2_destroy.restype = [vp], None
+        L.gpt2_checkpoint_read_config.argtypes = [ctypes.c_char_p, ctypes.POINTER(GPT2Config)]
+        L.gpt2_checkpoint_read_config.restype = ci
+        L.gpt2_build_from_checkpoint.argtypes = [ctypes.c_char_p]
+        L.gpt2_build_from_checkpoint.restype = vp
         L.gpt2_num_parameters.argtypes, L.gpt2_num_parameters.restype = [vp], cz
         L.gpt2_params_device.argtypes, L.gpt2_params_device.restype = [vp], vp
         L.gpt2_load_params_host.argtypes, L.gpt2_load_params_host.restype = [vp, vp, cz], ci
@@ -210,6 +215,14 @@ def argmax_forward(ids, logits, N, V):
     _check(lib().argmax_forward_status(_i32(ids), _f32(logits), N, V), "argmax_forward")
 
 
+def read_checkpoint_config(path) -> dict:
+    """Header of an llm.c checkpoint file as GPT2(**config) keywords (no GPU needed)."""
+    cfg = GPT2Config()
+    _check(lib().gpt2_checkpoint_read_config(os.fsencode(path), ctypes.byref(cfg)),
+           "gpt2_checkpoint_read_config")
+    return {name: getattr(cfg, name) for name, _ in GPT2Config._fields_}
+
+
 class Timer:
     """HIP-event timer on the null stream, the stream every launcher uses."""
 
@@ -236,13 +249,23 @@ class Timer:
 class GPT2:
     """The gpt2_forward driver (C++ side owns parameters and activations)."""
 
-    def __init__(self, *, max_seq_len, vocab_size, num_layers, num_heads, channels):
+    def __init__(self, *, max_seq_len, vocab_size, num_layers, num_heads, channels, _handle=None):
         self.config = GPT2Config(max_seq_len, vocab_size, num_layers, num_heads, channels)
-        self._h = lib().gpt2_create(ctypes.byref(self.config))
+        self._h = _handle or lib().gpt2_create(ctypes.byref(self.config))
         if not self._h:
             raise GPT2HipError("gpt2_create failed: " + lib().gpt2hip_last_error().decode())
         self.num_parameters = int(lib().gpt2_num_parameters(self._h))
         self._shape = None
+
+    @classmethod
+    def from_checkpoint(cls, path):
+        """Build from an llm.c fp32 checkpoint file (gpt2_124M.bin format)."""
+        cfg = read_checkpoint_config(path)
+        h = lib().gpt2_build_from_checkpoint(os.fsencode(path))
+        if not h:
+            raise GPT2HipError("gpt2_build_from_checkpoint failed: "
+                               + lib().gpt2hip_last_error().decode())
+        return cls(_handle=h, **cfg)
 
     def close(self):
         if getattr(self, "_h", None):

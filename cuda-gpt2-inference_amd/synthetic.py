@@ -58,3 +58,23 @@ def make_params(seed: int, *, perturb_affine: bool = False, **config) -> np.ndar
 def make_tokens(seed: int, B: int, T: int, vocab_size: int) -> np.ndarray:
     rng = np.random.default_rng(seed)
     return rng.integers(0, vocab_size, (B, T), dtype=np.int32)
+
+
+def write_llmc_checkpoint(path, flat_params: np.ndarray, *, version: int = 3, pad_to: int = 128,
+                          pad_value: float = 7.5, **config) -> None:
+    """Write parameters as an llm.c checkpoint file: 256 int32 header words, then fp32
+    tensors.  Version 3 pads wte's rows to a multiple of pad_to (filled with pad_value,
+    which a correct loader must never let through); version 1 does not pad."""
+    V, C = config["vocab_size"], config["channels"]
+    Vp = -(-V // pad_to) * pad_to if version == 3 else V
+    header = np.zeros(256, np.int32)
+    header[:7] = [20240326, version, config["max_seq_len"], V, config["num_layers"],
+                  config["num_heads"], C]
+    if version == 3:
+        header[7] = Vp
+    with open(path, "wb") as f:
+        f.write(header.tobytes())
+        f.write(np.ascontiguousarray(flat_params[:V * C], np.float32).tobytes())
+        if Vp > V:
+            f.write(np.full((Vp - V) * C, pad_value, np.float32).tobytes())
+        f.write(np.ascontiguousarray(flat_params[V * C:], np.float32).tobytes())
