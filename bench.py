@@ -220,6 +220,37 @@ def pmc_probe(g2):
     print(json.dumps({"pmc_probe": "done", "copy_bytes_each_way": src.numel() * 4}))
 
 
+def clock_probe(g2):
+    """Shader clocks per K slab and sustained clock frequency inside the GEMM kernel,
+    with zero and with N(0,1) operands (same instructions, different switching power)."""
+    import numpy as np
+    import torch
+    M = 8192
+    rows = []
+    for (C, OC) in ((768, 2304), (768, 768), (768, 3072), (3072, 768), (768, 50257)):
+        for data in ("zeros", "normal"):
+            x = torch.zeros(M, C, device="cuda") if data == "zeros" else torch.randn(M, C, device="cuda")
+            w = (torch.zeros(OC, C, device="cuda") if data == "zeros"
+                 else torch.randn(OC, C, device="cuda") * 0.02)
+            o = torch.empty(M, OC, device="cuda")
+            for _ in range(10):                       # bring the chip to its sustained state
+                g2.matmul_forward(o, x, w, None, 8, 1024, C, OC)
+            p = g2.matmul_forward_probe(o, x, w, None, 8, 1024, C, OC).astype(np.float64)
+            ns = (p[:, 1] - p[:, 0]) * 10.0
+            clk = p[:, 3] - p[:, 2]
+            nslab = C // 32
+            waves_per_simd = 2                        # both wave layouts put 2 waves on a SIMD
+            mfma_cycles = 64 * (128 * 192 // (32 * 32)) * 16 / 4   # per slab and SIMD: 6144
+            rows.append({"shape": f"M={M},C={C},OC={OC}", "operands": data,
+                         "workgroups": int(len(p)), "loop_us": float(ns.mean() / 1e3),
+                         "shader_clocks_per_slab": float(clk.mean() / nslab),
+                         "sustained_MHz": float(clk.sum() / ns.sum() * 1e3),
+                         "mfma_cycles_per_slab_one_workgroup": mfma_cycles})
+            log("  clock_probe", json.dumps(rows[-1]))
+            del x, w, o
+    print(json.dumps({"clock_probe": rows}))
+
+
 def cpu_baseline(model, cfg, B, T):
     """The CPU oracle on the host cores: one forward of the whole benchmark batch
     (a few seconds on 16 cores), after one untimed pass at B=1 to warm the threads."""
@@ -247,6 +278,8 @@ def main():
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--no-standalone", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="in-kernel wall/shader clock probe of the GEMM, zero vs normal operands")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="launch each kernel once plus a calibration copy (for rocprofv3 --pmc)")
     args = ap.parse_args()
@@ -266,6 +299,9 @@ def main():
 
     if args.pmc_probe:
         pmc_probe(g2)
+        return
+    if args.clock_probe:
+        clock_probe(g2)
         return
     cfg = dict(g2.GPT2_124M if args.model == "124M" else g2.GPT2_350M)
     B = args.batch or (8 if args.model == "124M" else 4)

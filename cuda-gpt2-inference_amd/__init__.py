@@ -38,7 +38,7 @@ EXPORTS = (
     "residual_forward", "residual_forward_status",
     "gelu_forward", "gelu_forward_status",
     "matmul_forward", "matmul_forward_status",
-    "matmul_forward_gelu", "matmul_forward_gelu_status",
+    "matmul_forward_gelu", "matmul_forward_gelu_status", "matmul_forward_probe_status",
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
     "gpt2_checkpoint_read_config", "gpt2_build_from_checkpoint",
@@ -108,6 +108,8 @@ def lib() -> ctypes.CDLL:
             f.argtypes, f.restype = args, None
             f = getattr(L, name + "_status")
             f.argtypes, f.restype = args, ci
+        L.matmul_forward_probe_status.argtypes = [vp] * 4 + [ci] * 4 + [vp, ci, ctypes.POINTER(ci)]
+        L.matmul_forward_probe_status.restype = ci
         L.gpt2_create.argtypes, L.gpt2_create.restype = [ctypes.POINTER(GPT2Config)], vp
         L.gpt2_destroy.argtypes, L.gpt2_destroy.restype = [vp], None
         L.gpt2_checkpoint_read_config.argtypes = [ctypes.c_char_p, ctypes.POINTER(GPT2Config)]
@@ -204,6 +206,20 @@ def matmul_forward(out, inp, weight, bias, B, T, C, OC):
 def matmul_forward_gelu(out, inp, weight, bias, B, T, C, OC, is_gelu):
     _check(lib().matmul_forward_gelu_status(_f32(out), _f32(inp), _f32(weight), _f32(bias), B, T,
                                             C, OC, int(bool(is_gelu))), "matmul_forward_gelu")
+
+
+def matmul_forward_probe(out, inp, weight, bias, B, T, C, OC):
+    """matmul_forward with the in-kernel clock probe.  Returns a (workgroups, 4) int64
+    array: wall clock (10 ns ticks) at K-loop start / end, shader clock at the same."""
+    import torch
+    cap = ((B * T + 127) // 128) * ((OC + 127) // 128)
+    probe = torch.zeros((cap, 4), dtype=torch.int64, device="cuda")
+    n = ctypes.c_int(0)
+    _check(lib().matmul_forward_probe_status(_f32(out), _f32(inp), _f32(weight), _f32(bias), B, T,
+                                             C, OC, probe.data_ptr(), cap, ctypes.byref(n)),
+           "matmul_forward_probe")
+    torch.cuda.synchronize()
+    return probe[:n.value].cpu().numpy()
 
 
 def attention_forward(out, qkvr, att, inp, B, T, C, NH):

@@ -24,6 +24,7 @@
 // a lane owns one output column, so the bias is folded into the accumulator's
 // initial value (as the reference does, 9_matmul_async_cg_tf32_gelu.cuh:56-84)
 // and every store instruction writes two 128-byte row segments.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.hpp"
@@ -286,10 +287,15 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
 
-template <int BM, int BN, int WGM, int WGN, bool GELU>
+// PROBE instantiations additionally record, per workgroup, the wall clock (100 MHz) and
+// the shader clock at the start and end of the slab loop: {wall0, wall1, clk0, clk1}
+// in probe[4*workgroup ..].  They tell MFMA issue efficiency (shader clocks per slab
+// against the 64 cycles per MFMA) apart from the clock frequency the chip sustains.
+template <int BM, int BN, int WGM, int WGN, bool GELU, bool PROBE = false>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn) {
+    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn,
+    unsigned long long* __restrict__ probe) {
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -449,12 +455,23 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   __builtin_amdgcn_s_waitcnt(0x0F70 | DMA_PER);  // vmcnt(DMA_PER): slab 0 has landed
   __syncthreads();
   read_ops(0, 0, 0);
+  unsigned long long wall0 = 0, clk0 = 0;
+  if (PROBE) {
+    wall0 = wall_clock64();
+    clk0 = clock64();
+  }
   int s = 0;
   for (; s + 1 < nslab; s += 2) {
     slab_body(s, std::integral_constant<int, 0>{});
     slab_body(s + 1, std::integral_constant<int, 1>{});
   }
   if (s < nslab) slab_body(s, std::integral_constant<int, 0>{});
+  if (PROBE && tid == 0) {
+    probe[4 * blockIdx.x + 0] = wall0;
+    probe[4 * blockIdx.x + 1] = wall_clock64();
+    probe[4 * blockIdx.x + 2] = clk0;
+    probe[4 * blockIdx.x + 3] = clock64();
+  }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // drain the (unused) DMAs before the LDS is released
 #undef G2_SGB
 #undef G2_READS_IN_SHADOW
@@ -506,22 +523,21 @@ __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const f
   out[idx] = gelu ? gelu_tanh(acc) : acc;
 }
 
-// Sets the dynamic-LDS limit of a kernel once per (thread, device, kernel).
-template <typename F>
-static int allow_lds(F kfn, size_t lds_bytes, int slot) {
+// Raises the dynamic-LDS limit of a kernel, once per (thread, device, kernel).
+static int allow_lds(const void* kfn, size_t lds_bytes) {
   static thread_local int configured_for = -1;
-  static thread_local unsigned configured_mask = 0;
+  static thread_local const void* configured[32];
+  static thread_local int nconfigured = 0;
   int dev = 0;
   G2_HIP(hipGetDevice(&dev));
   if (configured_for != dev) {
     configured_for = dev;
-    configured_mask = 0;
+    nconfigured = 0;
   }
-  if (!(configured_mask & (1u << slot))) {
-    G2_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    configured_mask |= 1u << slot;
-  }
+  for (int i = 0; i < nconfigured; i++)
+    if (configured[i] == kfn) return GPT2HIP_OK;
+  G2_HIP(hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  if (nconfigured < 32) configured[nconfigured++] = kfn;
   return GPT2HIP_OK;
 }
 
@@ -539,7 +555,7 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
                            : matmul_mfma_kernel<BM, BN, WGM, WGN, false, true>)
                    : (gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true, false>
                            : matmul_mfma_kernel<BM, BN, WGM, WGN, false, false>);
-  if (int rc = allow_lds(kfn, lds_bytes, (gelu ? 1 : 0) + (ktail ? 2 : 0))) return rc;
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
                      K, N, ntm, ntn);
   G2_LAUNCH_CHECK("matmul_forward");
@@ -547,25 +563,27 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
 }
 
 // LDS-DMA kernel: K % 32 == 0.
-template <int BM, int BN, int WGM, int WGN, int SLOT>
+template <int BM, int BN, int WGM, int WGN>
 static int launch_dma(float* out, const float* inp, const float* weight, const float* bias, int M,
-                      int K, int N, bool gelu) {
+                      int K, int N, bool gelu, unsigned long long* probe = nullptr) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
   const long long tiles = (long long)ntm * ntn;
   if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
-  auto kfn = gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true>
-                  : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
-  if (int rc = allow_lds(kfn, lds_bytes, SLOT + (gelu ? 1 : 0))) return rc;
+  auto kfn = probe ? matmul_dma_kernel<BM, BN, WGM, WGN, false, true>
+                   : gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true>
+                          : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
-                     K, N, ntm, ntn);
+                     K, N, ntm, ntn, probe);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
 
 static int matmul_dispatch(float* out, const float* inp, const float* weight, const float* bias,
-                           int B, int T, int C, int OC, bool gelu) {
+                           int B, int T, int C, int OC, bool gelu,
+                           unsigned long long* probe = nullptr, int* probe_groups = nullptr) {
   if (B < 0 || T < 0 || C < 1 || OC < 1)
     return fail(GPT2HIP_EINVAL, "matmul_forward: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
   const long long M64 = (long long)B * T;
@@ -574,6 +592,7 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
   if (M == 0) return GPT2HIP_OK;
   if (!out || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward: null pointer");
   if (C % 4 != 0 || !aligned16(inp) || !aligned16(weight)) {
+    if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs the MFMA path");
     const size_t total = (size_t)M * OC;
     hipLaunchKernelGGL(matmul_generic_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, 0,
                        out, inp, weight, bias, M, C, OC, gelu ? 1 : 0);
@@ -587,13 +606,17 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
     const long long t192 = (long long)((M + 127) / 128) * ((OC + 191) / 192);
     const long long t128 = (long long)((M + 127) / 128) * ((OC + 127) / 128);
     const long long cost192 = ((t192 + 255) / 256) * 3, cost128 = ((t128 + 255) / 256) * 2;
-    if (cost128 < cost192) return launch_dma<128, 128, 4, 2, 4>(out, inp, weight, bias, M, C, OC, gelu);
+    if (probe_groups) *probe_groups = (int)(cost128 < cost192 ? t128 : t192);
+    if (cost128 < cost192)
+      return launch_dma<128, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
     // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
     // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
     // gives every SIMD two waves to alternate between.
-    if (t192 >= 16 * 256) return launch_dma<128, 192, 2, 2, 0>(out, inp, weight, bias, M, C, OC, gelu);
-    return launch_dma<128, 192, 4, 2, 2>(out, inp, weight, bias, M, C, OC, gelu);
+    if (t192 >= 16 * 256)
+      return launch_dma<128, 192, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+    return launch_dma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
   }
+  if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs C %% 32 == 0");
   return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu);
 }
 
@@ -609,6 +632,20 @@ int matmul_forward_status(float* out, const float* inp, const float* weight, con
 void matmul_forward(float* out, const float* inp, const float* weight, const float* bias, int B,
                     int T, int C, int OC) {
   if (matmul_forward_status(out, inp, weight, bias, B, T, C, OC)) g2::die("matmul_forward");
+}
+
+int matmul_forward_probe_status(float* out, const float* inp, const float* weight,
+                                const float* bias, int B, int T, int C, int OC,
+                                unsigned long long* probe, int probe_capacity, int* workgroups) {
+  using namespace g2;
+  if (!probe || !workgroups) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: null pointer");
+  // dry run of the tile choice, to check the capacity before anything is launched
+  const long long t192 = (long long)(((long long)B * T + 127) / 128) * ((OC + 191) / 192);
+  const long long t128 = (long long)(((long long)B * T + 127) / 128) * ((OC + 127) / 128);
+  if (std::max(t192, t128) > probe_capacity)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_probe: probe buffer holds %d workgroups, need %lld",
+                probe_capacity, std::max(t192, t128));
+  return matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false, probe, workgroups);
 }
 
 int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,

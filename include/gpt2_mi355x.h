@@ -89,6 +89,17 @@ int matmul_forward_gelu_status(float* out, const float* inp, const float* weight
 void matmul_forward_gelu(float* out, const float* inp, const float* weight, const float* bias,
                          int B, int T, int C, int OC, int is_gelu);
 
+/* Diagnostic form of matmul_forward (C % 32 == 0, 16-byte aligned operands): the
+ * same kernel, which also stores for each of its workgroups four 64-bit words in
+ * probe[] (device memory, probe_capacity workgroups): wall clock (100 MHz) at the
+ * start and end of the K loop, then the shader clock at the same two instants.
+ * *workgroups receives the number of workgroups launched.  No counterpart in the
+ * reference; it separates instruction-issue efficiency from the clock frequency the
+ * chip sustains under the load. */
+int matmul_forward_probe_status(float* out, const float* inp, const float* weight,
+                                const float* bias, int B, int T, int C, int OC,
+                                unsigned long long* probe, int probe_capacity, int* workgroups);
+
 /* Causal multi-head self-attention.  inp is packed qkv (B,T,3C): q at column
  * 0, k at +C, v at +2C, head h at h*(C/NH) inside each; out is (B,T,C).
  * qkvr and att are the llm.c scratch arguments: ignored, may be NULL.  inp is

@@ -268,6 +268,42 @@ def test_matmul_identity_weight():
     assert np.array_equal(out.cpu().numpy(), b[None, :] + x)
 
 
+def test_matmul_probe_form_same_result_and_sane_clocks():
+    M, C, OC = 1024, 768, 768
+    x, w, b = mm_inputs(M, C, OC, 125)
+    ref = run_matmul(x, w, b)
+    out = torch.empty((M, OC), device="cuda")
+    p = g2.matmul_forward_probe(out, dev(x), dev(w), dev(b), 1, M, C, OC)
+    assert torch.equal(out, ref), "the probe instantiation must compute the same bits"
+    assert p.shape == (8 * 6, 4)                       # 128x128 tiles are chosen for this shape
+    wall = (p[:, 1] - p[:, 0]) * 10e-9                 # seconds
+    clk = p[:, 3] - p[:, 2]
+    assert (wall > 0).all() and (clk > 0).all()
+    per_slab = clk / (C // 32)
+    # one workgroup per CU here: a slab of a 128x128 tile is 4096 MFMA cycles per SIMD, so
+    # anything below that is impossible and anything far above means a broken pipeline
+    assert (per_slab >= 4096).all() and per_slab.mean() < 2 * 4096, per_slab.mean()
+    mhz = clk.sum() / wall.sum() / 1e6
+    assert 500 < mhz < 3000, mhz
+
+
+def test_matmul_probe_rejects_small_buffer_and_odd_k():
+    x, w, _ = mm_inputs(256, 64, 192, 126)
+    out = torch.empty((256, 192), device="cuda")
+    L = g2.lib()
+    import ctypes
+    probe = torch.zeros(4, dtype=torch.int64, device="cuda")
+    n = ctypes.c_int(0)
+    rc = L.matmul_forward_probe_status(out.data_ptr(), dev(x).data_ptr(), dev(w).data_ptr(), None,
+                                       1, 256, 64, 192, probe.data_ptr(), 1, ctypes.byref(n))
+    assert rc == 1 and b"probe buffer" in L.gpt2hip_last_error()
+    x2, w2, _ = mm_inputs(256, 36, 192, 127)             # K % 32 != 0: register-staged kernel
+    probe = torch.zeros(64, dtype=torch.int64, device="cuda")
+    rc = L.matmul_forward_probe_status(out.data_ptr(), dev(x2).data_ptr(), dev(w2).data_ptr(), None,
+                                       1, 256, 36, 192, probe.data_ptr(), 16, ctypes.byref(n))
+    assert rc == 1 and b"C % 32" in L.gpt2hip_last_error()
+
+
 # ------------------------------------------------------------------ attention
 @pytest.mark.parametrize("B,T,NH", [(8, 1024, 12), (8, 256, 12), (2, 1024, 16), (4, 256, 16),
                                     (4, 64, 12), (1, 1, 2), (2, 33, 3), (1, 130, 2), (1, 200, 1)])
