@@ -2,15 +2,20 @@
 // optional tanh-GELU epilogue.  True fp32 on the matrix cores
 // (v_mfma_f32_32x32x2_f32; gfx950 has no xf32 path).
 //
+// Three kernels share one tiling, LDS layout and MFMA mapping:
+//   matmul_dma_kernel      K % 32 == 0 (every GPT-2 shape): K slabs go from global
+//                          memory straight into LDS (global_load_lds_dwordx4)
+//   matmul_mfma_kernel     any K % 4 == 0: slabs staged through registers, K tail
+//                          zero-filled
+//   matmul_generic_kernel  anything else (K % 4 != 0, unaligned pointers)
+//
 // Tiling.  A workgroup owns a BM x BN output tile and walks K in slabs of
 // BK = 32.  Both operands are K-contiguous in memory ("NT" GEMM), so a slab of
-// either is rows of 32 floats = 8 chunks of 16 bytes.  Slabs are fetched with
-// 128-bit global loads into registers two slabs ahead, then stored to one of
-// two LDS buffers; one barrier per slab, placed inside the slab's MFMA work so
-// that no wave waits on a store->barrier->read chain.  In LDS, chunk c of row r sits at
-// chunk position c ^ (r & 7): eight lanes that read the same logical chunk of
-// eight consecutive rows then hit eight different 16-byte bank groups, which
-// makes both the 128-bit stores and the 128-bit operand reads conflict-free.
+// either is rows of 32 floats = 8 chunks of 16 bytes, held in one of two LDS
+// buffers; there is one barrier per slab, placed inside the slab's MFMA work so
+// that no wave waits on a fill->barrier->read chain.  In LDS, chunk c of row r sits
+// at chunk position c ^ (r & 7): eight lanes that read the same logical chunk of
+// eight consecutive rows then hit eight different 16-byte bank groups.
 //
 // MFMA operand mapping.  v_mfma_f32_32x32x2_f32 takes A[i][k] from lane
 // (i = lane%32, k = lane/32) and B[k][j] from lane (j = lane%32, k = lane/32).
@@ -24,6 +29,12 @@
 // a lane owns one output column, so the bias is folded into the accumulator's
 // initial value (as the reference does, 9_matmul_async_cg_tf32_gelu.cuh:56-84)
 // and every store instruction writes two 128-byte row segments.
+//
+// What bounds it.  Measured with the in-kernel clock probe below: a slab of a
+// 128x192 tile costs 6363 shader clocks against 6144 cycles of MFMA work (96.6 %
+// issue efficiency); the shader clock itself sits at 2.0-2.2 GHz under this kernel
+// with N(0,1) operands and at 2.25-2.35 GHz with all-zero operands, i.e. the chip's
+// power management, not the instruction stream, sets the distance to the 2.4 GHz peak.
 #include <algorithm>
 #include <type_traits>
 
