@@ -183,6 +183,25 @@ def standalone(g2):
     out.append({"kernel": "layernorm_forward", "shape": f"N={M},C={C}", "ms": ms,
                 "GB/s": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS,
                 "note": "rotating 16 buffer sets, 768 MiB"})
+    # encoder gather and argmax at the forward's sizes
+    V = 50257
+    wte = torch.randn(V, C, device=dev) * 0.02
+    wpe = torch.randn(1024, C, device=dev) * 0.01
+    ids = torch.randint(0, V, (8, 1024), dtype=torch.int32, device=dev)
+    args = [(P(o[k]), P(ids), P(wte), P(wpe), 8, 1024, C) for k in range(16)]
+    ms = time_launch(g2, lambda i: L.encoder_forward(*args[i % 16]), iters=96, warmup=16)
+    nb = 4 * M + 8 * M * C + 4 * 1024 * C
+    out.append({"kernel": "encoder_forward", "shape": f"B=8,T=1024,C={C}", "ms": ms,
+                "GB/s": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS})
+    del x, o, wte
+    logits = torch.randn(M, V, device=dev)
+    am = torch.empty(M, dtype=torch.int32, device=dev)
+    a = (P(am), P(logits), M, V)
+    ms = time_launch(g2, lambda i: L.argmax_forward(*a), iters=10, warmup=3)
+    nb = 4 * M * V + 4 * M
+    out.append({"kernel": "argmax_forward", "shape": f"N={M},V={V}", "ms": ms,
+                "GB/s": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS,
+                "note": "1.65 GB of logits: larger than the Infinity Cache"})
     return out
 
 
