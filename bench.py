@@ -295,6 +295,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--model", choices=("124M", "350M"), default="124M")
     ap.add_argument("--batch", type=int, default=None)
+    ap.add_argument("--seq-len", type=int, default=1024)
     ap.add_argument("--no-standalone", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--clock-probe", action="store_true",
@@ -324,7 +325,7 @@ def main():
         return
     cfg = dict(g2.GPT2_124M if args.model == "124M" else g2.GPT2_350M)
     B = args.batch or (8 if args.model == "124M" else 4)
-    T = 1024
+    T = args.seq_len
     model = g2.GPT2(**cfg)
     init_params_on_device(model, syn, cfg, seed=1337)
     ids = torch.randint(0, cfg["vocab_size"], (B, T), dtype=torch.int32, device="cuda")
@@ -379,7 +380,8 @@ def main():
     achieved = dom_flops / dom_ms / 1e9
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
                 "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-                "traffic": DOMINANT_TRAFFIC_BYTES if (args.model == "124M" and B == 8) else None,
+                "traffic": (DOMINANT_TRAFFIC_BYTES
+                            if (args.model == "124M" and B == 8 and T == 1024) else None),
                 "kernel": "matmul_dma_kernel<128,192,4,2,false>",
                 "avg_launch_ms": dom_ms, "flops_per_launch": dom_flops,
                 "launches_per_forward": dom_launches}

@@ -212,7 +212,7 @@ def matmul_forward_probe(out, inp, weight, bias, B, T, C, OC):
     """matmul_forward with the in-kernel clock probe.  Returns a (workgroups, 4) int64
     array: wall clock (10 ns ticks) at K-loop start / end, shader clock at the same."""
     import torch
-    cap = ((B * T + 127) // 128) * ((OC + 127) // 128)
+    cap = ((B * T + 31) // 32) * ((OC + 31) // 32)
     probe = torch.zeros((cap, 4), dtype=torch.int64, device="cuda")
     n = ctypes.c_int(0)
     _check(lib().matmul_forward_probe_status(_f32(out), _f32(inp), _f32(weight), _f32(bias), B, T,

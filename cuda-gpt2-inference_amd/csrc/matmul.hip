@@ -612,20 +612,42 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
   }
   // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
   if (C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31)) {
-    // Tile choice by wave quantisation over the 256 CUs: time ~ rounds x tile area.
-    // 128x192 wins ties (fewer LDS reads per MFMA).
-    const long long t192 = (long long)((M + 127) / 128) * ((OC + 191) / 192);
-    const long long t128 = (long long)((M + 127) / 128) * ((OC + 127) / 128);
-    const long long cost192 = ((t192 + 255) / 256) * 3, cost128 = ((t128 + 255) / 256) * 2;
-    if (probe_groups) *probe_groups = (int)(cost128 < cost192 ? t128 : t192);
-    if (cost128 < cost192)
-      return launch_dma<128, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
-    // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
-    // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
-    // gives every SIMD two waves to alternate between.
-    if (t192 >= 16 * 256)
-      return launch_dma<128, 192, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
-    return launch_dma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+    // Tile choice by wave quantisation over the 256 CUs: estimated time ~ (tiles per
+    // CU, rounded up) x tile area / efficiency of that tile shape (smaller tiles spend
+    // more LDS reads and DMA loads per MFMA).  Large problems end up on 128x192; small
+    // M (short prompts, small batches) on 64x64 or 32x32 tiles that still fill the chip.
+    struct Cand { int bm, bn; double eff; };
+    const Cand cands[] = {{128, 192, 1.00}, {128, 128, 0.97}, {64, 64, 0.80}, {32, 32, 0.50}};
+    int best = 0;
+    double best_cost = 0;
+    long long best_tiles = 0;
+    for (int i = 0; i < 4; i++) {
+      const long long t = (long long)((M + cands[i].bm - 1) / cands[i].bm) *
+                          ((OC + cands[i].bn - 1) / cands[i].bn);
+      const double cost = (double)((t + 255) / 256) * cands[i].bm * cands[i].bn / cands[i].eff;
+      if (i == 0 || cost < best_cost) {
+        best = i;
+        best_cost = cost;
+        best_tiles = t;
+      }
+    }
+    if (best_tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
+    if (probe_groups) *probe_groups = (int)best_tiles;
+    switch (best) {
+      case 3:
+        return launch_dma<32, 32, 1, 1>(out, inp, weight, bias, M, C, OC, gelu, probe);
+      case 2:
+        return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+      case 1:
+        return launch_dma<128, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+      default:
+        // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
+        // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
+        // gives every SIMD two waves to alternate between.
+        if (best_tiles >= 16 * 256)
+          return launch_dma<128, 192, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+        return launch_dma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+    }
   }
   if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs C %% 32 == 0");
   return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu);
@@ -650,12 +672,11 @@ int matmul_forward_probe_status(float* out, const float* inp, const float* weigh
                                 unsigned long long* probe, int probe_capacity, int* workgroups) {
   using namespace g2;
   if (!probe || !workgroups) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: null pointer");
-  // dry run of the tile choice, to check the capacity before anything is launched
-  const long long t192 = (long long)(((long long)B * T + 127) / 128) * ((OC + 191) / 192);
-  const long long t128 = (long long)(((long long)B * T + 127) / 128) * ((OC + 127) / 128);
-  if (std::max(t192, t128) > probe_capacity)
+  // the smallest tile shape bounds the number of workgroups any choice can launch
+  const long long most = (((long long)B * T + 31) / 32) * ((OC + 31) / 32);
+  if (most > probe_capacity)
     return fail(GPT2HIP_EINVAL, "matmul_forward_probe: probe buffer holds %d workgroups, need %lld",
-                probe_capacity, std::max(t192, t128));
+                probe_capacity, most);
   return matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false, probe, workgroups);
 }
 

@@ -93,7 +93,8 @@ void matmul_forward_gelu(float* out, const float* inp, const float* weight, cons
  * same kernel, which also stores for each of its workgroups four 64-bit words in
  * probe[] (device memory, probe_capacity workgroups): wall clock (100 MHz) at the
  * start and end of the K loop, then the shader clock at the same two instants.
- * *workgroups receives the number of workgroups launched.  No counterpart in the
+ * *workgroups receives the number of workgroups launched (at most
+ * ceil(B*T/32) * ceil(OC/32), which probe_capacity must cover).  No counterpart in the
  * reference; it separates instruction-issue efficiency from the clock frequency the
  * chip sustains under the load. */
 int matmul_forward_probe_status(float* out, const float* inp, const float* weight,

@@ -275,14 +275,14 @@ def test_matmul_probe_form_same_result_and_sane_clocks():
     out = torch.empty((M, OC), device="cuda")
     p = g2.matmul_forward_probe(out, dev(x), dev(w), dev(b), 1, M, C, OC)
     assert torch.equal(out, ref), "the probe instantiation must compute the same bits"
-    assert p.shape == (8 * 6, 4)                       # 128x128 tiles are chosen for this shape
+    assert p.shape == (16 * 12, 4)                     # 64x64 tiles are chosen for this shape
     wall = (p[:, 1] - p[:, 0]) * 10e-9                 # seconds
     clk = p[:, 3] - p[:, 2]
     assert (wall > 0).all() and (clk > 0).all()
     per_slab = clk / (C // 32)
-    # one workgroup per CU here: a slab of a 128x128 tile is 4096 MFMA cycles per SIMD, so
-    # anything below that is impossible and anything far above means a broken pipeline
-    assert (per_slab >= 4096).all() and per_slab.mean() < 2 * 4096, per_slab.mean()
+    # one workgroup per CU here: a slab of a 64x64 tile is 16 MFMAs = 1024 cycles on each
+    # SIMD, so anything below that is impossible; far above means a broken pipeline
+    assert (per_slab >= 1024).all() and per_slab.mean() < 3 * 1024, per_slab.mean()
     mhz = clk.sum() / wall.sum() / 1e6
     assert 500 < mhz < 3000, mhz
 
@@ -292,15 +292,15 @@ def test_matmul_probe_rejects_small_buffer_and_odd_k():
     out = torch.empty((256, 192), device="cuda")
     L = g2.lib()
     import ctypes
-    probe = torch.zeros(4, dtype=torch.int64, device="cuda")
+    probe = torch.zeros(4 * 47, dtype=torch.int64, device="cuda")
     n = ctypes.c_int(0)
     rc = L.matmul_forward_probe_status(out.data_ptr(), dev(x).data_ptr(), dev(w).data_ptr(), None,
-                                       1, 256, 64, 192, probe.data_ptr(), 1, ctypes.byref(n))
+                                       1, 256, 64, 192, probe.data_ptr(), 47, ctypes.byref(n))
     assert rc == 1 and b"probe buffer" in L.gpt2hip_last_error()
     x2, w2, _ = mm_inputs(256, 36, 192, 127)             # K % 32 != 0: register-staged kernel
-    probe = torch.zeros(64, dtype=torch.int64, device="cuda")
+    probe = torch.zeros(4 * 48, dtype=torch.int64, device="cuda")
     rc = L.matmul_forward_probe_status(out.data_ptr(), dev(x2).data_ptr(), dev(w2).data_ptr(), None,
-                                       1, 256, 36, 192, probe.data_ptr(), 16, ctypes.byref(n))
+                                       1, 256, 36, 192, probe.data_ptr(), 48, ctypes.byref(n))
     assert rc == 1 and b"C % 32" in L.gpt2hip_last_error()
 
 
