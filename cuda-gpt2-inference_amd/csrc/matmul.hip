@@ -2,9 +2,11 @@
 // optional tanh-GELU epilogue.  True fp32 on the matrix cores
 // (v_mfma_f32_32x32x2_f32; gfx950 has no xf32 path).
 //
-// Three kernels share one tiling, LDS layout and MFMA mapping:
+// Four kernels share one tiling, LDS layout and MFMA mapping:
 //   matmul_dma_kernel      K % 32 == 0 (every GPT-2 shape): K slabs go from global
 //                          memory straight into LDS (global_load_lds_dwordx4)
+//   matmul_ring_kernel     the same for problems of few small tiles (short prompts):
+//                          deeper slab ring, optional K split between a tile's waves
 //   matmul_mfma_kernel     any K % 4 == 0: slabs staged through registers, K tail
 //                          zero-filled
 //   matmul_generic_kernel  anything else (K % 4 != 0, unaligned pointers)
@@ -518,6 +520,195 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   }
 }
 
+// s_waitcnt immediate that waits until at most n vector-memory operations of this wave
+// are outstanding and waits for nothing else (vmcnt is split over bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+
+// Small problems (few output tiles): same LDS layout, DMA fill and MFMA mapping as
+// matmul_dma_kernel, organised for latency instead of issue rate.  With one small tile
+// per CU there is too little MFMA work per slab to cover a memory round trip, so the
+// slabs go through a ring of NBUF buffers with NBUF-1 fills in flight, and the waves of
+// a workgroup can also split K (KS): wave set ks takes k-groups ks*4/KS .. of every
+// slab, so a 32x32 tile still keeps all four SIMDs of its CU busy.  The partial
+// accumulators are summed through LDS in a fixed order (ks = 0, 1, ...), so results do
+// not depend on timing.
+template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool GELU>
+__global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
+    float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
+    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn) {
+  constexpr int NMN = WGM * WGN;
+  constexpr int NW = NMN * KS;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_PER = BM / 8 / NW, B_PER = BN / 8 / NW;
+  constexpr int DMA_PER = A_PER + B_PER;
+  constexpr int GPW = 4 / KS;  // k-groups of a slab per wave
+  static_assert(BM / 8 % NW == 0 && BN / 8 % NW == 0, "tile/waves mismatch");
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be 32x32 MFMA tiles");
+  static_assert(KS == 1 || KS == 2 || KS == 4, "K split must divide the 4 k-groups");
+  static_assert(NBUF >= 2 && (NBUF - 1) * DMA_PER < 64, "vmcnt is a 6-bit counter");
+  constexpr int STAGE_BYTES = (BM + BN) * CHUNKS * 16;
+  static_assert((KS - 1) * NMN * TM * TN * 16 * 64 * 4 <= NBUF * STAGE_BYTES,
+                "the K-split reduction reuses the ring's LDS");
+
+  extern __shared__ f32x4 lds[];  // [NBUF][(BM + BN) * CHUNKS]: A rows then B rows
+  char* const lds_bytes = reinterpret_cast<char*>(lds);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ks = wave / NMN, wmn = wave % NMN;
+  const int wm = wmn / WGN, wn = wmn % WGN;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, ntm, ntn, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // LDS-DMA descriptors, as in matmul_dma_kernel
+  const char* const a_tile = reinterpret_cast<const char*>(inp + (size_t)m0 * K);
+  const char* const b_tile = reinterpret_cast<const char*>(weight + (size_t)n0 * K);
+  unsigned dma_off[DMA_PER];
+  int dma_group[DMA_PER];
+  {
+    const int rr = lane >> 3, c = (lane & 7) ^ rr;
+#pragma unroll
+    for (int j = 0; j < DMA_PER; j++) {
+      if (j < A_PER) {
+        dma_group[j] = wave * A_PER + j;
+        const int row = 8 * dma_group[j] + rr;
+        dma_off[j] = (unsigned)((min(m0 + row, M - 1) - m0) * K + c * 4) * 4u;
+      } else {
+        dma_group[j] = BM / 8 + wave * B_PER + (j - A_PER);
+        const int row = 8 * (dma_group[j] - BM / 8) + rr;
+        dma_off[j] = (unsigned)((min(n0 + row, N - 1) - n0) * K + c * 4) * 4u;
+      }
+    }
+  }
+  const int nslab = K / BK;
+  auto dma_slab = [&](int slab, int buf) {
+    const size_t kbytes = (size_t)min(slab, nslab - 1) * (BK * 4);  // past the end: reload
+    const char* a_k = a_tile + kbytes;
+    const char* b_k = b_tile + kbytes;
+    asm volatile("" : "+s"(a_k), "+s"(b_k));  // keep the scalar-base addressing form
+#pragma unroll
+    for (int j = 0; j < DMA_PER; j++)
+      __builtin_amdgcn_global_load_lds(
+          (glb_void_t*)((j < A_PER ? a_k : b_k) + dma_off[j]),
+          (lds_void_t*)(lds_bytes + buf * STAGE_BYTES + dma_group[j] * 1024), 16, 0, 0);
+  };
+#pragma unroll
+  for (int i = 0; i < NBUF - 1; i++) dma_slab(i, i);
+
+  // accumulators: wave set 0 starts from the bias of the lane's column, the others from 0
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int col = n0 + wn * WN + j * 32 + (lane & 31);
+    const float bv = (bias != nullptr && ks == 0 && col < N) ? bias[col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = bv;
+  }
+
+  const int h = lane >> 5;
+  const int sw = lane & 7;
+  int a_addr[GPW], b_addr[GPW];
+#pragma unroll
+  for (int i = 0; i < GPW; i++) {
+    const int g = ks * GPW + i;
+    a_addr[i] = ((wm * WM + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw)) * 16;
+    b_addr[i] = (BM * CHUNKS + (wn * WN + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw)) * 16;
+  }
+
+  // Slab s lives in buffer s % NBUF.  Per slab: wait for this wave's fills of slab s,
+  // BARRIER (every wave's fills of slab s have landed and every wave has finished with
+  // slab s-1), refill slab s-1's buffer with slab s+NBUF-1, multiply slab s.
+  int buf = 0;
+  for (int s = 0; s < nslab; s++) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only((NBUF - 2) * DMA_PER));
+    __syncthreads();
+    dma_slab(s + NBUF - 1, buf == 0 ? NBUF - 1 : buf - 1);
+    const char* const stage = lds_bytes + buf * STAGE_BYTES;
+#pragma unroll
+    for (int g = 0; g < GPW; g++) {
+      f32x4 af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+        af[i] = *reinterpret_cast<const f32x4*>(stage + a_addr[g] + i * (32 * BK * 4));
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+        bf[j] = *reinterpret_cast<const f32x4*>(stage + b_addr[g] + j * (32 * BK * 4));
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+    }
+    buf = buf + 1 == NBUF ? 0 : buf + 1;
+  }
+  __builtin_amdgcn_s_waitcnt(vmcnt_only(0));  // drain the (unused) fills past the last slab
+
+  if (KS > 1) {
+    // sum the wave sets' partial tiles: [ks-1][wmn][tile][v][lane], lane-contiguous
+    __syncthreads();  // every wave is done with the ring
+    float* const red = reinterpret_cast<float*>(lds);
+    if (ks > 0) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int v = 0; v < 16; v++)
+            red[((((ks - 1) * NMN + wmn) * (TM * TN) + i * TN + j) * 16 + v) * 64 + lane] =
+                acc[i][j][v];
+    }
+    __syncthreads();
+    if (ks > 0) return;
+#pragma unroll
+    for (int k2 = 1; k2 < KS; k2++)
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int v = 0; v < 16; v++)
+            acc[i][j][v] +=
+                red[((((k2 - 1) * NMN + wmn) * (TM * TN) + i * TN + j) * 16 + v) * 64 + lane];
+  }
+
+  const bool full = (m0 + BM <= M) && (n0 + BN <= N);
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int col = n0 + wn * WN + j * 32 + (lane & 31);
+      const int rbase = m0 + wm * WM + i * 32 + 4 * h;
+      float* o = out + (size_t)rbase * N + col;
+      if (full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          float r = acc[i][j][v];
+          if (GELU) r = gelu_tanh(r);
+          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
+        }
+      } else if (col < N) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int row = rbase + 8 * (v >> 2) + (v & 3);
+          if (row < M) {
+            float r = acc[i][j][v];
+            if (GELU) r = gelu_tanh(r);
+            out[(size_t)row * N + col] = r;
+          }
+        }
+      }
+    }
+  }
+}
+
 // Any shape, any alignment; one thread per output.  Only used when K is not a
 // multiple of 4 or an operand is not 16-byte aligned.
 __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const float* inp,
@@ -592,6 +783,24 @@ static int launch_dma(float* out, const float* inp, const float* weight, const f
   return GPT2HIP_OK;
 }
 
+// Ring kernel for small problems: K % 32 == 0.
+template <int BM, int BN, int WGM, int WGN, int KS, int NBUF>
+static int launch_ring(float* out, const float* inp, const float* weight, const float* bias, int M,
+                       int K, int N, bool gelu) {
+  constexpr int NT = WGM * WGN * KS * kWave;
+  constexpr size_t lds_bytes = (size_t)NBUF * (BM + BN) * BK * sizeof(float);
+  const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
+  const long long tiles = (long long)ntm * ntn;
+  if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
+  auto kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true>
+                  : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false>;
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
+                     K, N, ntm, ntn);
+  G2_LAUNCH_CHECK("matmul_forward");
+  return GPT2HIP_OK;
+}
+
 static int matmul_dispatch(float* out, const float* inp, const float* weight, const float* bias,
                            int B, int T, int C, int OC, bool gelu,
                            unsigned long long* probe = nullptr, int* probe_groups = nullptr) {
@@ -612,16 +821,19 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
   }
   // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
   if (C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31)) {
-    // Tile choice by wave quantisation over the 256 CUs: estimated time ~ (tiles per
-    // CU, rounded up) x tile area / efficiency of that tile shape (smaller tiles spend
-    // more LDS reads and DMA loads per MFMA).  Large problems end up on 128x192; small
-    // M (short prompts, small batches) on 64x64 or 32x32 tiles that still fill the chip.
+    // Tile choice.  Measured over M = 64 .. 8192 at the GPT-2 shapes, a launch takes
+    // about  fixed + ceil(tiles / 256 CUs) x (tile area x K) / (per-CU MFMA rate x eff)
+    // with eff = 1 / 0.985 / 0.89 / 0.77 for the four tile shapes (smaller tiles move
+    // more bytes into LDS per MFMA), so the tile with the least
+    // ceil(tiles / 256) x area / eff wins: 128x192 for large problems, 64x64 or 32x32
+    // for short prompts and small batches, where they still fill the chip.  The clock
+    // probe exists for the two large shapes only.
     struct Cand { int bm, bn; double eff; };
-    const Cand cands[] = {{128, 192, 1.00}, {128, 128, 0.97}, {64, 64, 0.80}, {32, 32, 0.50}};
+    const Cand cands[] = {{128, 192, 1.00}, {128, 128, 0.985}, {64, 64, 0.89}, {32, 32, 0.77}};
     int best = 0;
     double best_cost = 0;
     long long best_tiles = 0;
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < (probe ? 2 : 4); i++) {
       const long long t = (long long)((M + cands[i].bm - 1) / cands[i].bm) *
                           ((OC + cands[i].bn - 1) / cands[i].bn);
       const double cost = (double)((t + 255) / 256) * cands[i].bm * cands[i].bn / cands[i].eff;
@@ -635,9 +847,13 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
     if (probe_groups) *probe_groups = (int)best_tiles;
     switch (best) {
       case 3:
-        return launch_dma<32, 32, 1, 1>(out, inp, weight, bias, M, C, OC, gelu, probe);
+        // one 32x32 tile per workgroup, its four waves splitting K
+        return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu);
       case 2:
-        return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+        // up to two tiles per CU: latency-bound, ring of four slabs and a 2-way K split
+        if (best_tiles <= 2 * 256)
+          return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu);
+        return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu);
       case 1:
         return launch_dma<128, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
       default:

@@ -216,6 +216,7 @@ def run_matmul(x, w, b, gelu=None):
     (8192, 768, 2304), (8192, 768, 768), (8192, 768, 3072), (8192, 3072, 768),   # GPT-2 124M
     (256, 768, 2304), (256, 3072, 768),                                          # B=4, T=64
     (4096, 1024, 3072), (4096, 4096, 1024),                                      # GPT-2 350M
+    (4096, 768, 768), (1024, 1024, 1024), (1000, 96, 1000), (64, 768, 3072),     # 64x64 / 32x32 tiles
     (128, 32, 192), (1, 4, 1), (130, 36, 200), (77, 100, 81), (300, 768, 50),    # edges
 ])
 def test_matmul_bias(M, C, OC):
@@ -269,20 +270,20 @@ def test_matmul_identity_weight():
 
 
 def test_matmul_probe_form_same_result_and_sane_clocks():
-    M, C, OC = 1024, 768, 768
+    M, C, OC = 2048, 768, 3072                         # 16 x 16 tiles of 128x192: one per CU
     x, w, b = mm_inputs(M, C, OC, 125)
     ref = run_matmul(x, w, b)
     out = torch.empty((M, OC), device="cuda")
     p = g2.matmul_forward_probe(out, dev(x), dev(w), dev(b), 1, M, C, OC)
     assert torch.equal(out, ref), "the probe instantiation must compute the same bits"
-    assert p.shape == (16 * 12, 4)                     # 64x64 tiles are chosen for this shape
+    assert p.shape == (16 * 16, 4)
     wall = (p[:, 1] - p[:, 0]) * 10e-9                 # seconds
     clk = p[:, 3] - p[:, 2]
     assert (wall > 0).all() and (clk > 0).all()
     per_slab = clk / (C // 32)
-    # one workgroup per CU here: a slab of a 64x64 tile is 16 MFMAs = 1024 cycles on each
-    # SIMD, so anything below that is impossible; far above means a broken pipeline
-    assert (per_slab >= 1024).all() and per_slab.mean() < 3 * 1024, per_slab.mean()
+    # a slab of a 128x192 tile is 384 MFMAs = 6144 cycles on each of the CU's four SIMDs,
+    # so anything below that is impossible; far above means a broken pipeline
+    assert (per_slab >= 6144).all() and per_slab.mean() < 2 * 6144, per_slab.mean()
     mhz = clk.sum() / wall.sum() / 1e6
     assert 500 < mhz < 3000, mhz
 
