@@ -202,6 +202,22 @@ def standalone(g2):
     out.append({"kernel": "argmax_forward", "shape": f"N={M},V={V}", "ms": ms,
                 "GB/s": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS,
                 "note": "1.65 GB of logits: larger than the Infinity Cache"})
+    # lm-head + argmax: two launches through the logits buffer against the fused launcher
+    x = torch.randn(M, C, device=dev)
+    wte = torch.randn(V, C, device=dev) * 0.02
+    a_mm = (P(logits), P(x), P(wte), None, 8, 1024, C, V)
+    def unfused(i):
+        L.matmul_forward(*a_mm)
+        L.argmax_forward(*a)
+    ms_unfused = time_launch(g2, unfused, iters=8, warmup=2)
+    need = L.matmul_forward_argmax_workspace(8, 1024, V)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    a_f = (P(am), P(ws), need, P(x), P(wte), None, 8, 1024, C, V)
+    ms_fused = time_launch(g2, lambda i: L.matmul_forward_argmax_status(*a_f), iters=8, warmup=2)
+    tf = 2.0 * M * C * V / ms_fused / 1e9
+    out.append({"kernel": "matmul_forward_argmax", "shape": f"M={M},C={C},OC={V}", "ms": ms_fused,
+                "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS,
+                "note": f"matmul_forward + argmax_forward through 1.65 GB of logits: {ms_unfused:.3f} ms"})
     return out
 
 

@@ -41,10 +41,12 @@ EXPORTS = (
     "matmul_forward_gelu", "matmul_forward_gelu_status", "matmul_forward_probe_status",
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
+    "matmul_forward_argmax_workspace", "matmul_forward_argmax_status",
     "gpt2_checkpoint_read_config", "gpt2_build_from_checkpoint",
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
-    "gpt2_forward_device_status", "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
+    "gpt2_forward_device_status", "gpt2_forward_argmax_status",
+    "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
     "gpt2hip_timer_stop_ms",
 )
@@ -124,6 +126,12 @@ def lib() -> ctypes.CDLL:
         L.gpt2_forward_status.argtypes, L.gpt2_forward_status.restype = [vp, vp, ci, ci], ci
         L.gpt2_forward_device_status.argtypes = [vp, vp, ci, ci]
         L.gpt2_forward_device_status.restype = ci
+        L.gpt2_forward_argmax_status.argtypes = [vp, vp, ci, ci, vp]
+        L.gpt2_forward_argmax_status.restype = ci
+        L.matmul_forward_argmax_workspace.argtypes = [ci, ci, ci]
+        L.matmul_forward_argmax_workspace.restype = cz
+        L.matmul_forward_argmax_status.argtypes = [vp, vp, cz, vp, vp, vp, ci, ci, ci, ci]
+        L.matmul_forward_argmax_status.restype = ci
         L.gpt2_forward_profiled_status.argtypes = [vp, vp, ci, ci, ctypes.POINTER(ctypes.c_float)]
         L.gpt2_forward_profiled_status.restype = ci
         L.gpt2_logits.argtypes, L.gpt2_logits.restype = [vp], vp
@@ -231,6 +239,18 @@ def argmax_forward(ids, logits, N, V):
     _check(lib().argmax_forward_status(_i32(ids), _f32(logits), N, V), "argmax_forward")
 
 
+def matmul_forward_argmax(ids, inp, weight, bias, B, T, C, OC, workspace=None):
+    """ids (B*T int32) = per-row argmax of inp . weight^T + bias, without storing the product.
+    workspace: optional uint8 CUDA tensor of matmul_forward_argmax_workspace(B, T, OC) bytes."""
+    import torch
+    need = lib().matmul_forward_argmax_workspace(B, T, OC)
+    if workspace is None:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
+    _check(lib().matmul_forward_argmax_status(_i32(ids), workspace.data_ptr(), workspace.numel(),
+                                              _f32(inp), _f32(weight), _f32(bias), B, T, C, OC),
+           "matmul_forward_argmax")
+
+
 def read_checkpoint_config(path) -> dict:
     """Header of an llm.c checkpoint file as GPT2(**config) keywords (no GPU needed)."""
     cfg = GPT2Config()
@@ -313,6 +333,16 @@ class GPT2:
         else:
             _check(lib().gpt2_forward_device_status(self._h, _i32(inputs), B, T), "gpt2_forward")
         self._shape = (B, T)
+
+    def forward_argmax(self, inputs_device):
+        """Forward that keeps only each position's argmax token id; returns (B,T) int32."""
+        import torch
+        B, T = inputs_device.shape
+        ids = torch.empty((B, T), dtype=torch.int32, device="cuda")
+        _check(lib().gpt2_forward_argmax_status(self._h, _i32(inputs_device), B, T,
+                                                ids.data_ptr()), "gpt2_forward_argmax")
+        self._shape = (B, T)
+        return ids
 
     def forward_profiled(self, inputs_device):
         """Forward with per-launch HIP events; returns {category: ms} for this pass."""

@@ -73,6 +73,15 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// (value, index) combination of an argmax: the larger value wins, the smaller index
+// among equal values.  NaN never wins (every comparison with it is false).
+// Written with selects: as branches, a chain of these turns into divergent control flow.
+__device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int oi) {
+  const bool take = (ov > v) | ((ov == v) & (oi < i));
+  v = take ? ov : v;
+  i = take ? oi : i;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
   v = fmaxf(v, dpp<0xB1>(v));
   v = fmaxf(v, dpp<0x4E>(v));
@@ -95,5 +104,10 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 #endif
+
+// encoder_forward with an optional on-device check of the token ids against the
+// vocabulary size V (V = 0: ids are trusted, as the reference trusts them).
+int encoder_launch(float* out, const int* inp, const float* wte, const float* wpe, int B, int T,
+                   int C, int V);
 
 }  // namespace g2

@@ -8,28 +8,40 @@ namespace g2 {
 constexpr int kBlock = 256;
 
 // ---- encoder: out[b,t,:] = wte[ids[b,t],:] + wpe[t,:] ----------------------
-// One thread per float4 of the output; the token id is a broadcast load.
+// One thread per float4 of the output; the token id is a broadcast load.  With V > 0 an
+// id outside [0, V) is not dereferenced: its row is filled with NaN instead, which shows
+// in everything computed from it.
 __global__ __launch_bounds__(kBlock) void encoder_vec_kernel(
     f32x4* __restrict__ out, const int* __restrict__ ids, const f32x4* __restrict__ wte,
-    const f32x4* __restrict__ wpe, int T, int C4, size_t total4) {
+    const f32x4* __restrict__ wpe, int T, int C4, size_t total4, int V) {
   const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= total4) return;
   const size_t bt = i / C4;
   const int c = (int)(i - bt * C4);
   const int t = (int)(bt % T);
   const int id = ids[bt];
+  if (V > 0 && (unsigned)id >= (unsigned)V) {
+    const float q = __builtin_nanf("");
+    out[i] = f32x4{q, q, q, q};
+    return;
+  }
   out[i] = wte[(size_t)id * C4 + c] + wpe[(size_t)t * C4 + c];
 }
 
 __global__ __launch_bounds__(kBlock) void encoder_scalar_kernel(
     float* __restrict__ out, const int* __restrict__ ids, const float* __restrict__ wte,
-    const float* __restrict__ wpe, int T, int C, size_t total) {
+    const float* __restrict__ wpe, int T, int C, size_t total, int V) {
   const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= total) return;
   const size_t bt = i / C;
   const int c = (int)(i - bt * C);
   const int t = (int)(bt % T);
-  out[i] = wte[(size_t)ids[bt] * C + c] + wpe[(size_t)t * C + c];
+  const int id = ids[bt];
+  if (V > 0 && (unsigned)id >= (unsigned)V) {
+    out[i] = __builtin_nanf("");
+    return;
+  }
+  out[i] = wte[(size_t)id * C + c] + wpe[(size_t)t * C + c];
 }
 
 // ---- residual / gelu -----------------------------------------------------
@@ -110,13 +122,6 @@ static int launch_map(const char* name, float* out, const float* inp1, const flo
 // ascending index order (so "first maximum" is kept with a strict >), then
 // (value, index) pairs are reduced with "larger value, or equal value and
 // smaller index".
-__device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int oi) {
-  if (ov > v || (ov == v && oi < i)) {
-    v = ov;
-    i = oi;
-  }
-}
-
 __global__ __launch_bounds__(kBlock) void argmax_rows_kernel(int* __restrict__ ids,
                                                               const float* __restrict__ logits,
                                                               int V) {
@@ -156,13 +161,9 @@ __global__ __launch_bounds__(kBlock) void argmax_rows_kernel(int* __restrict__ i
   }
 }
 
-}  // namespace g2
-
-extern "C" {
-
-int encoder_forward_status(float* out, const int* inp, const float* wte, const float* wpe, int B,
-                           int T, int C) {
-  using namespace g2;
+// V > 0: token ids are checked against the vocabulary size on the device (see the kernels).
+int encoder_launch(float* out, const int* inp, const float* wte, const float* wpe, int B, int T,
+                   int C, int V) {
   if (B < 0 || T < 0 || C < 1) return fail(GPT2HIP_EINVAL, "encoder_forward: bad shape B=%d T=%d C=%d", B, T, C);
   const size_t total = (size_t)B * T * C;
   if (total == 0) return GPT2HIP_OK;
@@ -172,13 +173,22 @@ int encoder_forward_status(float* out, const int* inp, const float* wte, const f
     hipLaunchKernelGGL(encoder_vec_kernel, dim3((unsigned)((total4 + kBlock - 1) / kBlock)),
                        dim3(kBlock), 0, 0, reinterpret_cast<f32x4*>(out), inp,
                        reinterpret_cast<const f32x4*>(wte), reinterpret_cast<const f32x4*>(wpe), T,
-                       C / 4, total4);
+                       C / 4, total4, V);
   } else {
     hipLaunchKernelGGL(encoder_scalar_kernel, dim3((unsigned)((total + kBlock - 1) / kBlock)),
-                       dim3(kBlock), 0, 0, out, inp, wte, wpe, T, C, total);
+                       dim3(kBlock), 0, 0, out, inp, wte, wpe, T, C, total, V);
   }
   G2_LAUNCH_CHECK("encoder_forward");
   return GPT2HIP_OK;
+}
+
+}  // namespace g2
+
+extern "C" {
+
+int encoder_forward_status(float* out, const int* inp, const float* wte, const float* wpe, int B,
+                           int T, int C) {
+  return g2::encoder_launch(out, inp, wte, wpe, B, T, C, 0);
 }
 
 void encoder_forward(float* out, const int* inp, const float* wte, const float* wpe, int B, int T,

@@ -44,17 +44,23 @@ struct GPT2 {
   float* proj;     // (M,C) attproj / fcproj output
   float* fch;      // (M,4C) gelu(fc)
   float* logits;   // (M,V)
+  void* pairs;     // workspace of matmul_forward_argmax for (M,V)
+  size_t pairs_bytes;
   int last_B, last_T;
+  bool last_has_logits;
 };
 
 namespace g2 {
 
 static void free_activations(GPT2* m) {
-  void* ptrs[] = {m->ids, m->res_a, m->res_b, m->ln, m->qkv, m->atty, m->proj, m->fch, m->logits};
+  void* ptrs[] = {m->ids,  m->res_a, m->res_b, m->ln,     m->qkv,
+                  m->atty, m->proj,  m->fch,   m->logits, m->pairs};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   m->ids = nullptr;
   m->res_a = m->res_b = m->ln = m->qkv = m->atty = m->proj = m->fch = m->logits = nullptr;
+  m->pairs = nullptr;
+  m->pairs_bytes = 0;
   m->cap_tokens = 0;
 }
 
@@ -77,7 +83,8 @@ static int reserve(GPT2* m, int B, int T) {
       {(void**)&m->res_b, n * C * 4},              {(void**)&m->ln, n * C * 4},
       {(void**)&m->qkv, n * 3 * C * 4},            {(void**)&m->atty, n * C * 4},
       {(void**)&m->proj, n * C * 4},               {(void**)&m->fch, n * 4 * C * 4},
-      {(void**)&m->logits, n * V * 4}};
+      {(void**)&m->logits, n * V * 4},
+      {&m->pairs, matmul_forward_argmax_workspace(1, (int)M, (int)V)}};
   for (auto& w : want) {
     hipError_t e = hipMalloc(w.p, w.bytes);
     if (e != hipSuccess) {
@@ -87,6 +94,7 @@ static int reserve(GPT2* m, int B, int T) {
                   hipGetErrorString(e));
     }
   }
+  m->pairs_bytes = matmul_forward_argmax_workspace(1, (int)M, (int)V);
   m->cap_tokens = M;
   return GPT2HIP_OK;
 }
@@ -110,8 +118,10 @@ struct Profile {
   }
 };
 
-// The forward pass proper; ids are already in m->ids.
-static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr) {
+// The forward pass proper; ids are already in m->ids.  With next_ids the lm-head keeps
+// only the argmax of every row (written there) and m->logits is left untouched.
+static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
+                            int* next_ids = nullptr) {
   const GPT2Config& c = m->cfg;
   const int C = c.channels, L = c.num_layers, NH = c.num_heads, V = c.vocab_size;
   const size_t cs = (size_t)C;
@@ -129,7 +139,7 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr) {
 
   float* residual = m->res_a;  // current residual stream
   float* other = m->res_b;
-  G2_STEP(GPT2_PROF_ENCODER, encoder_forward_status(residual, m->ids, P(P_WTE), P(P_WPE), B, T, C));
+  G2_STEP(GPT2_PROF_ENCODER, encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE), B, T, C, V));
   // the one stand-alone layernorm: ln1 of layer 0
   G2_STEP(GPT2_PROF_LAYERNORM, layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, T, C));
   for (int l = 0; l < L; l++) {
@@ -153,11 +163,16 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr) {
                                                    m->proj, nw, nb, B, T, C));
   }
   // lm-head: weight-tied to wte, no bias, unpadded vocabulary
-  G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_status(m->logits, m->ln, P(P_WTE), nullptr, B, T, C, V));
+  if (next_ids)
+    G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_argmax_status(next_ids, m->pairs, m->pairs_bytes, m->ln,
+                                                                  P(P_WTE), nullptr, B, T, C, V));
+  else
+    G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_status(m->logits, m->ln, P(P_WTE), nullptr, B, T, C, V));
 #undef G2_STEP
 #undef G2_TRY
   m->last_B = B;
   m->last_T = T;
+  m->last_has_logits = next_ids == nullptr;
   return GPT2HIP_OK;
 }
 
@@ -331,6 +346,17 @@ int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int
   return forward_resident(model, B, T);
 }
 
+int gpt2_forward_argmax_status(GPT2* model, const int* inputs_device, int B, int T,
+                               int* next_ids_device) {
+  using namespace g2;
+  if (int rc = reserve(model, B, T)) return rc;
+  if (!inputs_device || !next_ids_device)
+    return fail(GPT2HIP_EINVAL, "gpt2_forward_argmax: null pointer");
+  G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
+                        hipMemcpyDeviceToDevice, 0));
+  return forward_resident(model, B, T, nullptr, next_ids_device);
+}
+
 int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, int T,
                                  float* ms_per_category) {
   using namespace g2;
@@ -356,8 +382,8 @@ const float* gpt2_lnf(const GPT2* model) { return model ? model->ln : nullptr; }
 
 int gpt2_argmax_status(GPT2* model, int* ids_device) {
   using namespace g2;
-  if (!model || !model->logits || model->last_B == 0)
-    return fail(GPT2HIP_EINVAL, "gpt2_argmax: no forward pass has run");
+  if (!model || !model->logits || model->last_B == 0 || !model->last_has_logits)
+    return fail(GPT2HIP_EINVAL, "gpt2_argmax: no forward pass has left logits");
   return argmax_forward_status(ids_device, model->logits, model->last_B * model->last_T,
                                model->cfg.vocab_size);
 }

@@ -65,6 +65,43 @@ __device__ __forceinline__ void tile_of_block(int pid, int ntm, int ntn, int& tm
   }
 }
 
+// Argmax over the 32 lanes of a half-wave for N rows at once: bv[e] / bx[e] are this
+// lane's (value, column) candidates for rows e = 0..N-1, the same rows in every lane.
+// Butterfly over lane bits 4..0 (OFF = 16..1).  While a lane still holds more rows than
+// the exchange distance, partners split the rows between them (each keeps one half of
+// the list and hands the other half over), so the work halves at every step and, for
+// N = 32, lane l ends up with the finished pair of row l alone; 32 lanes reducing every
+// row five times would cost five times the cross-lane traffic.  On return the lane holds
+// max(N / 32, 1) rows starting at row `first`; lanes with writer == false hold duplicates.
+template <int N, int OFF>
+__device__ __forceinline__ void argmax_fold(float* bv, int* bx, int lane, int& first,
+                                            bool& writer) {
+  if constexpr (OFF >= 1) {
+    const bool up = (lane & OFF) != 0;
+    if constexpr (N > OFF) {
+      constexpr int HN = N / 2;
+#pragma unroll
+      for (int e = 0; e < HN; e++) {
+        float kv = up ? bv[e + HN] : bv[e];
+        int ki = up ? bx[e + HN] : bx[e];
+        const float sv = up ? bv[e] : bv[e + HN];
+        const int si = up ? bx[e] : bx[e + HN];
+        argmax_combine(kv, ki, __shfl_xor(sv, OFF, 64), __shfl_xor(si, OFF, 64));
+        bv[e] = kv;
+        bx[e] = ki;
+      }
+      first += up ? HN : 0;
+      argmax_fold<HN, OFF / 2>(bv, bx, lane, first, writer);
+    } else {
+#pragma unroll
+      for (int e = 0; e < N; e++)
+        argmax_combine(bv[e], bx[e], __shfl_xor(bv[e], OFF, 64), __shfl_xor(bx[e], OFF, 64));
+      writer = writer && !up;
+      argmax_fold<N, OFF / 2>(bv, bx, lane, first, writer);
+    }
+  }
+}
+
 template <int BM, int BN, int WGM, int WGN, bool GELU, bool KTAIL>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
@@ -304,11 +341,16 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 // the shader clock at the start and end of the slab loop: {wall0, wall1, clk0, clk1}
 // in probe[4*workgroup ..].  They tell MFMA issue efficiency (shader clocks per slab
 // against the 64 cycles per MFMA) apart from the clock frequency the chip sustains.
-template <int BM, int BN, int WGM, int WGN, bool GELU, bool PROBE = false>
+//
+// ARGMAX: instead of storing the tile, every wave reduces its part of each output row to
+// one (largest value, its column) pair and stores that in out[row][tn * WGN + wn] (the
+// value) and arg_idx[row][tn * WGN + wn] (the column): ntn * WGN pairs per row, which
+// argmax_pairs_kernel reduces.  The (M, N) product itself never reaches memory.
+template <int BM, int BN, int WGM, int WGN, bool GELU, bool PROBE = false, bool ARGMAX = false>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
     const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn,
-    unsigned long long* __restrict__ probe) {
+    unsigned long long* __restrict__ probe, int* __restrict__ arg_idx) {
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -490,6 +532,47 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
 #undef G2_READS_IN_SHADOW
 
   // ---- epilogue -----------------------------------------------------------
+  if (ARGMAX) {
+    const size_t pairs = (size_t)ntn * WGN;
+    const size_t slot = (size_t)tn * WGN + wn;
+    // This lane's best over its own columns, for each of its R rows (ascending columns:
+    // a strict > keeps the first maximum).
+    constexpr int R = TM * 16;
+    float bv[R];
+    int bx[R];
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const int col = n0 + wn * WN + j * 32 + (lane & 31);
+          const float a = acc[i][j][v];
+          const bool take = (col < N) & (a > best);
+          best = take ? a : best;
+          bi = take ? col : bi;
+        }
+        bv[i * 16 + v] = best;
+        bx[i * 16 + v] = bi;
+      }
+    }
+    int first = 0;
+    bool writer = true;
+    argmax_fold<R, 16>(bv, bx, lane, first, writer);
+    constexpr int n = R > 32 ? R / 32 : 1;  // rows a lane ends up with
+#pragma unroll
+    for (int e = 0; e < n; e++) {
+      const int r = first + e;  // index i * 16 + v of the row this lane finished
+      const int row = m0 + wm * WM + (r >> 4) * 32 + 4 * h + 8 * ((r & 15) >> 2) + (r & 3);
+      if (writer && row < M) {
+        out[(size_t)row * pairs + slot] = bv[e];
+        arg_idx[(size_t)row * pairs + slot] = bx[e];
+      }
+    }
+    return;
+  }
   const bool full = (m0 + BM <= M) && (n0 + BN <= N);
 #pragma unroll
   for (int i = 0; i < TM; i++) {
@@ -725,6 +808,67 @@ __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const f
   out[idx] = gelu ? gelu_tanh(acc) : acc;
 }
 
+// Reduces the (value, column) pairs that the ARGMAX form of matmul_dma_kernel leaves
+// per row to the row's argmax; one wave per row, four rows per block.
+__global__ __launch_bounds__(256) void argmax_pairs_kernel(int* __restrict__ ids,
+                                                            const float* __restrict__ val,
+                                                            const int* __restrict__ idx, int M,
+                                                            int pairs) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int lane = threadIdx.x & 63;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int p = lane; p < pairs; p += 64)
+    argmax_combine(best, bi, val[(size_t)row * pairs + p], idx[(size_t)row * pairs + p]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    argmax_combine(best, bi, ov, oi);
+  }
+  // a row of all -inf / NaN never beats the initial value: report index 0
+  if (lane == 0) ids[row] = (bi == 0x7fffffff) ? 0 : bi;
+}
+
+// Any shape, any alignment: one block per row computes the row's products one thread per
+// column (the arithmetic of matmul_generic_kernel) and keeps only their argmax.
+__global__ __launch_bounds__(256) void matmul_argmax_generic_kernel(int* __restrict__ ids,
+                                                                     const float* inp,
+                                                                     const float* weight,
+                                                                     const float* bias, int K,
+                                                                     int N) {
+  const float* x = inp + (size_t)blockIdx.x * K;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int col = threadIdx.x; col < N; col += 256) {
+    const float* w = weight + (size_t)col * K;
+    float acc = bias ? bias[col] : 0.f;
+    for (int k = 0; k < K; k++) acc += x[k] * w[k];
+    if (acc > best) {
+      best = acc;
+      bi = col;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(best, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    argmax_combine(best, bi, ov, oi);
+  }
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  if ((threadIdx.x & 63) == 0) {
+    sv[threadIdx.x >> 6] = best;
+    si[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; w++) argmax_combine(best, bi, sv[w], si[w]);
+    ids[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+  }
+}
+
 // Raises the dynamic-LDS limit of a kernel, once per (thread, device, kernel).
 static int allow_lds(const void* kfn, size_t lds_bytes) {
   static thread_local int configured_for = -1;
@@ -778,8 +922,28 @@ static int launch_dma(float* out, const float* inp, const float* weight, const f
                           : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
-                     K, N, ntm, ntn, probe);
+                     K, N, ntm, ntn, probe, (int*)nullptr);
   G2_LAUNCH_CHECK("matmul_forward");
+  return GPT2HIP_OK;
+}
+
+// The 128x192 LDS-DMA kernel in its ARGMAX form followed by the pair reduction.
+constexpr int kArgmaxBN = 192, kArgmaxWGN = 2;
+template <int WGM>
+static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const float* inp,
+                             const float* weight, const float* bias, int M, int K, int N) {
+  constexpr int BM = 128, BN = kArgmaxBN, WGN = kArgmaxWGN;
+  constexpr int NT = WGM * WGN * kWave;
+  constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
+  const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
+  auto kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, false, true>;
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
+  hipLaunchKernelGGL(kfn, dim3((unsigned)(ntm * ntn)), dim3(NT), lds_bytes, 0, pair_val, inp, weight,
+                     bias, M, K, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx);
+  G2_LAUNCH_CHECK("matmul_forward_argmax");
+  hipLaunchKernelGGL(argmax_pairs_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, 0, ids,
+                     pair_val, pair_idx, M, ntn * WGN);
+  G2_LAUNCH_CHECK("matmul_forward_argmax");
   return GPT2HIP_OK;
 }
 
@@ -894,6 +1058,43 @@ int matmul_forward_probe_status(float* out, const float* inp, const float* weigh
     return fail(GPT2HIP_EINVAL, "matmul_forward_probe: probe buffer holds %d workgroups, need %lld",
                 probe_capacity, most);
   return matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false, probe, workgroups);
+}
+
+size_t matmul_forward_argmax_workspace(int B, int T, int OC) {
+  if (B < 1 || T < 1 || OC < 1) return 0;
+  const size_t pairs = (size_t)((OC + g2::kArgmaxBN - 1) / g2::kArgmaxBN) * g2::kArgmaxWGN;
+  return (size_t)B * T * pairs * 8;
+}
+
+int matmul_forward_argmax_status(int* ids, void* workspace, size_t workspace_bytes, const float* inp,
+                                 const float* weight, const float* bias, int B, int T, int C,
+                                 int OC) {
+  using namespace g2;
+  if (B < 0 || T < 0 || C < 1 || OC < 1)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
+  const long long M64 = (long long)B * T;
+  if (M64 > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: B*T too large");
+  const int M = (int)M64;
+  if (M == 0) return GPT2HIP_OK;
+  if (!ids || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: null pointer");
+  if (C % BK != 0 || !aligned16(inp) || !aligned16(weight) ||
+      (long long)C * 192 * 4 >= (1LL << 31)) {
+    hipLaunchKernelGGL(matmul_argmax_generic_kernel, dim3((unsigned)M), dim3(256), 0, 0, ids, inp,
+                       weight, bias, C, OC);
+    G2_LAUNCH_CHECK("matmul_forward_argmax");
+    return GPT2HIP_OK;
+  }
+  const size_t need = matmul_forward_argmax_workspace(B, T, OC);
+  if (!workspace || workspace_bytes < need)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: workspace of %zu bytes, need %zu",
+                workspace_bytes, need);
+  const long long tiles = (long long)((M + 127) / 128) * ((OC + 191) / 192);
+  if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: too many tiles");
+  float* pair_val = static_cast<float*>(workspace);
+  int* pair_idx = reinterpret_cast<int*>(pair_val + need / 8);
+  if (tiles >= 16 * 256)
+    return launch_dma_argmax<2>(ids, pair_val, pair_idx, inp, weight, bias, M, C, OC);
+  return launch_dma_argmax<4>(ids, pair_val, pair_idx, inp, weight, bias, M, C, OC);
 }
 
 int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,

@@ -117,6 +117,20 @@ void attention_forward(float* out, float* qkvr, float* att, const float* inp, in
 int argmax_forward_status(int* ids, const float* logits, int N, int V);
 void argmax_forward(int* ids, const float* logits, int N, int V);
 
+/* matmul_forward followed by argmax_forward without the (B*T, OC) product ever reaching
+ * memory: ids[r] = argmax_o (inp[r,:] . weight[o,:] + bias[o]), lowest index wins ties.
+ * For C % 32 == 0 and 16-byte aligned operands (the lm-head) the GEMM's tiles are reduced
+ * to (value, column) pairs in their epilogue and a second small kernel reduces the pairs;
+ * the result equals argmax_forward over matmul_forward's output exactly.  workspace is
+ * device memory of at least matmul_forward_argmax_workspace(B, T, OC) bytes.  Other shapes
+ * take a slow one-block-per-row kernel and ignore the workspace.  No counterpart in the
+ * reference, which runs its matmul launcher (kernels/matmul/2_matmul_cublas.cuh:34) and
+ * reads all logits back. */
+size_t matmul_forward_argmax_workspace(int B, int T, int OC);
+int matmul_forward_argmax_status(int* ids, void* workspace, size_t workspace_bytes, const float* inp,
+                                 const float* weight, const float* bias, int B, int T, int C,
+                                 int OC);
+
 /* ---- whole model: the gpt2_forward driver (llm.c train_gpt2_fp32.cu's
  * gpt2_forward, which the reference plugs its kernels into, README.md:19;
  * dataflow in reference images/gpt2/gpt2_flow.png). ---- */
@@ -161,10 +175,17 @@ int gpt2_reserve(GPT2* model, int B, int T);
 
 /* Forward pass.  gpt2_forward takes HOST token ids like llm.c and copies them
  * in; gpt2_forward_device takes ids already on the device.  Afterwards
- * gpt2_logits() is (B,T,V) on the device.  Launches are asynchronous. */
+ * gpt2_logits() is (B,T,V) on the device.  Launches are asynchronous.  Host ids
+ * outside [0, vocab_size) are rejected; device ids are checked by the first kernel,
+ * which fills the rows of bad ids with NaN instead of reading outside the table. */
 int gpt2_forward_status(GPT2* model, const int* inputs_host, int B, int T);
 void gpt2_forward(GPT2* model, const int* inputs_host, int B, int T);
 int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int T);
+/* Forward pass that keeps only the argmax of every position's logits (greedy next
+ * token ids, B*T ints on the device): the lm-head runs as matmul_forward_argmax, the
+ * logits buffer is not written and gpt2_argmax_status is unavailable afterwards. */
+int gpt2_forward_argmax_status(GPT2* model, const int* inputs_device, int B, int T,
+                               int* next_ids_device);
 /* The same forward pass with a HIP event recorded on the null stream around
  * every launch; waits for completion and adds each launch's elapsed ms into
  * ms_per_category[GPT2_PROF_COUNT] (host memory).  No counterpart in the

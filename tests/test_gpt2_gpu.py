@@ -81,6 +81,47 @@ def test_gpt2_350M_B1_T128():
     check(*run_both(dict(g2.GPT2_350M), 1, 128, seed=21))
 
 
+def test_gpt2_forward_argmax_matches_forward_then_argmax():
+    for cfg, B, T in ((dict(g2.GPT2_124M), 2, 128),
+                      (dict(max_seq_len=80, vocab_size=331, num_layers=2, num_heads=2, channels=128),
+                       3, 77)):
+        print(f"gpt2 forward_argmax cfg={cfg} B={B} T={T}", flush=True)
+        params = syn.make_params(31, perturb_affine=True, **cfg)
+        ids = torch.from_numpy(syn.make_tokens(32, B, T, cfg["vocab_size"])).cuda()
+        model = g2.GPT2(**cfg)
+        try:
+            model.load_params(params)
+            model.forward(ids)
+            want = model.argmax().clone()
+            model.logits().fill_(float("nan"))          # the fused pass must not need them
+            got = model.forward_argmax(ids)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want)
+            assert torch.isnan(model.logits()).all(), "forward_argmax must not write logits"
+            with pytest.raises(g2.GPT2HipError):
+                model.argmax()                          # no logits were left by that pass
+        finally:
+            model.close()
+
+
+def test_gpt2_device_ids_outside_vocabulary_give_nan_rows_not_faults():
+    cfg = dict(max_seq_len=16, vocab_size=50, num_layers=1, num_heads=1, channels=64)
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(syn.make_params(41, **cfg))
+        ids = syn.make_tokens(42, 3, 8, 50)
+        ids[1, 3] = 50
+        ids[0, 5] = -1
+        model.forward(torch.from_numpy(ids).cuda())
+        torch.cuda.synchronize()
+        bad = torch.isnan(model.logits()).all(-1).cpu().numpy()
+        # a NaN row shows at its own and every later position of its sequence (earlier
+        # positions of that sequence are unspecified); other sequences are untouched
+        assert bad[0, 5:].all() and bad[1, 3:].all() and not bad[2].any()
+    finally:
+        model.close()
+
+
 def test_gpt2_rejects_bad_inputs():
     model = g2.GPT2(max_seq_len=16, vocab_size=50, num_layers=1, num_heads=1, channels=64)
     try:

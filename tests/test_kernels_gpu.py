@@ -385,6 +385,57 @@ def test_argmax_bit_exact(N, V):
     assert np.array_equal(ids.cpu().numpy(), oracle.argmax_forward(x))
 
 
+# ------------------------------------------------------------------ fused matmul + argmax
+@pytest.mark.parametrize("M,C,OC,bias", [
+    (8192, 768, 50257, False),      # the lm-head: 4-wave tiles, ragged last column tile
+    (256, 768, 50257, False),       # 8-wave tiles
+    (300, 64, 1000, True),          # ragged rows and columns, bias
+    (128, 32, 192, True),           # a single K slab, exactly one column tile
+    (70, 36, 81, True),             # K % 32 != 0: one-block-per-row kernel
+    (33, 30, 17, False),            # K % 4 != 0
+])
+def test_matmul_argmax_equals_unfused(M, C, OC, bias):
+    say(f"matmul+argmax M={M} C={C} OC={OC}")
+    x, w, b = mm_inputs(M, C, OC, 141, bias=bias)
+    db = dev(b) if bias else None
+    full, ids, pad = guard((M,), torch.int32)
+    g2.matmul_forward_argmax(ids, dev(x), dev(w), db, 1, M, C, OC)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    got = ids.cpu().numpy()
+    logits = torch.empty((M, OC), device="cuda")
+    g2.matmul_forward(logits, dev(x), dev(w), db, 1, M, C, OC)
+    if C % 32 == 0:
+        # same accumulators as matmul_forward: exactly the argmax of its output
+        unfused = torch.empty(M, dtype=torch.int32, device="cuda")
+        g2.argmax_forward(unfused, logits, M, OC)
+        assert np.array_equal(got, unfused.cpu().numpy())
+    # against the oracle on a row subset: the chosen column's oracle value is the oracle's
+    # maximum up to the matmul tolerance (an exact tie-break is only defined per backend)
+    rows = np.unique(np.linspace(0, M - 1, 96).astype(np.int64))
+    exp = oracle.matmul_forward(x[rows], w, b)
+    chosen = exp[np.arange(len(rows)), got[rows]]
+    assert (exp.max(-1) - chosen <= 1e-5 + 1e-4 * np.abs(exp.max(-1))).all()
+
+
+def test_matmul_argmax_ties_nan_and_workspace_check():
+    M, C, OC = 64, 32, 400
+    x = np.zeros((M, C), np.float32)
+    w = np.zeros((OC, C), np.float32)
+    b = np.zeros(OC, np.float32)
+    b[[7, 200, 399]] = 2.0          # three equal maxima in different tiles and waves: lowest wins
+    x[1, 0] = np.nan                # a row of NaN products: nothing beats the start, index 0
+    ids = torch.full((M,), -1, dtype=torch.int32, device="cuda")
+    g2.matmul_forward_argmax(ids, dev(x), dev(w), dev(b), 1, M, C, OC)
+    got = ids.cpu().numpy()
+    assert got[0] == 7 and got[1] == 0 and (got[2:] == 7).all()
+    need = g2.lib().matmul_forward_argmax_workspace(1, M, OC)
+    assert need == M * 3 * 2 * 8     # 3 column tiles x 2 waves along N x (value, index)
+    small = torch.empty(need - 1, dtype=torch.uint8, device="cuda")
+    with pytest.raises(g2.GPT2HipError, match="workspace"):
+        g2.matmul_forward_argmax(ids, dev(x), dev(w), dev(b), 1, M, C, OC, workspace=small)
+
+
 # ------------------------------------------------------------------ error paths
 def test_bad_shapes_raise_and_leave_the_device_usable():
     a = torch.zeros(64, device="cuda")
