@@ -81,6 +81,27 @@ def test_gpt2_350M_B1_T128():
     check(*run_both(dict(g2.GPT2_350M), 1, 128, seed=21))
 
 
+def test_gpt2_against_committed_float64_fixture():
+    from golden import load_gpt2_tiny
+    cfg, params, ids, exp_logits, exp_lnf = load_gpt2_tiny()
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(params)
+        model.forward(ids)
+        torch.cuda.synchronize()
+        logits = model.logits().cpu().numpy()
+        lnf = model.lnf().cpu().numpy()
+        am = model.argmax().cpu().numpy()
+    finally:
+        model.close()
+    print(f"  fixture: max|dlogits|={np.abs(logits - exp_logits).max():.3e}", flush=True)
+    assert np.abs(lnf - exp_lnf).max() < 2e-5
+    assert np.abs(logits - exp_logits).max() < 2e-5
+    top2 = np.sort(exp_logits, -1)[..., -2:]
+    clear = (top2[..., 1] - top2[..., 0]) > 1e-4
+    assert np.array_equal(am[clear], exp_logits.argmax(-1)[clear])
+
+
 def test_gpt2_forward_argmax_matches_forward_then_argmax():
     for cfg, B, T in ((dict(g2.GPT2_124M), 2, 128),
                       (dict(max_seq_len=80, vocab_size=331, num_layers=2, num_heads=2, channels=128),

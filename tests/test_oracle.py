@@ -313,6 +313,19 @@ def test_gpt2_forward_tiny_float64():
     assert np.array_equal(am, logits.argmax(-1))
 
 
+def test_gpt2_forward_against_committed_float64_fixture():
+    from golden import load_gpt2_tiny
+    cfg, params, ids, exp_logits, exp_lnf = load_gpt2_tiny()
+    logits, am, lnf = oracle.gpt2_forward(params, ids, maxT=cfg["max_seq_len"], V=cfg["vocab_size"],
+                                          L=cfg["num_layers"], NH=cfg["num_heads"],
+                                          C=cfg["channels"], want_lnf=True)
+    assert np.abs(lnf - exp_lnf).max() < 2e-5
+    assert np.abs(logits - exp_logits).max() < 2e-5
+    top2 = np.sort(exp_logits, -1)[..., -2:]
+    clear = (top2[..., 1] - top2[..., 0]) > 1e-4
+    assert np.array_equal(am[clear], exp_logits.argmax(-1)[clear])
+
+
 def test_param_count_124M():
     assert oracle.num_parameters(1024, 50257, 12, 768) == 124_439_808
     assert oracle.num_parameters(1024, 50257, 24, 1024) == 354_823_168
