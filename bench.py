@@ -314,6 +314,8 @@ def main():
     ap.add_argument("--seq-len", type=int, default=1024)
     ap.add_argument("--no-standalone", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the forward pass replayed from a HIP graph")
     ap.add_argument("--clock-probe", action="store_true",
                     help="in-kernel wall/shader clock probe of the GEMM, zero vs normal operands")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -361,6 +363,18 @@ def main():
     log(f"forward {args.model} B={B} T={T}: {ms_per_step:.3f} ms/step, {tokens_per_s:,.0f} tok/s"
         f" (logits finite: {finite})")
 
+    graph_ms = None
+    if args.graph:
+        for _ in range(max(args.warmup, 2)):          # the first call captures
+            model.forward_graph(ids)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            model.forward_graph(ids)
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        log(f"  replayed from a HIP graph: {graph_ms:.3f} ms/step")
+
     # the same K steps again with a HIP event around every launch
     prof = {k: 0.0 for k in g2.PROF_CATEGORIES}
     for _ in range(args.steps):
@@ -398,7 +412,8 @@ def main():
                 "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                 "traffic": (DOMINANT_TRAFFIC_BYTES
                             if (args.model == "124M" and B == 8 and T == 1024) else None),
-                "kernel": "matmul_dma_kernel<128,192,4,2,false>",
+                "kernel": ("matmul_dma_kernel<128,192,4,2,false>" if B * T == 8192 else
+                           "matmul_forward, qkv / attproj / fcproj launches (tile shape by size)"),
                 "avg_launch_ms": dom_ms, "flops_per_launch": dom_flops,
                 "launches_per_forward": dom_launches}
 
@@ -414,6 +429,8 @@ def main():
         "forward_frac_fp32_mfma": (sum(flops.values()) / (ms_per_step * 1e9)) / PEAK_FP32_MFMA_TFLOPS,
         "kernels": kernels,
     }
+    if graph_ms is not None:
+        result["graph_replay_ms_per_step"] = graph_ms
     if not args.no_standalone:
         result["standalone"] = standalone(g2)
         for r in result["standalone"]:

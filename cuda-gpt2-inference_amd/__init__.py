@@ -31,7 +31,7 @@ HIPCC_FLAGS = (
 )
 
 EXPORTS = (
-    "gpt2hip_last_error",
+    "gpt2hip_last_error", "gpt2hip_set_stream", "gpt2hip_get_stream",
     "encoder_forward", "encoder_forward_status",
     "layernorm_forward", "layernorm_forward_status",
     "fused_residual_layernorm_forward", "fused_residual_layernorm_forward_status",
@@ -45,7 +45,8 @@ EXPORTS = (
     "gpt2_checkpoint_read_config", "gpt2_build_from_checkpoint",
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
-    "gpt2_forward_device_status", "gpt2_forward_argmax_status",
+    "gpt2_forward_device_status", "gpt2_forward_graph_status",
+    "gpt2_forward_argmax_status",
     "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
     "gpt2hip_timer_stop_ms",
@@ -126,6 +127,10 @@ def lib() -> ctypes.CDLL:
         L.gpt2_forward_status.argtypes, L.gpt2_forward_status.restype = [vp, vp, ci, ci], ci
         L.gpt2_forward_device_status.argtypes = [vp, vp, ci, ci]
         L.gpt2_forward_device_status.restype = ci
+        L.gpt2_forward_graph_status.argtypes = [vp, vp, ci, ci]
+        L.gpt2_forward_graph_status.restype = ci
+        L.gpt2hip_set_stream.argtypes, L.gpt2hip_set_stream.restype = [vp], None
+        L.gpt2hip_get_stream.argtypes, L.gpt2hip_get_stream.restype = [], vp
         L.gpt2_forward_argmax_status.argtypes = [vp, vp, ci, ci, vp]
         L.gpt2_forward_argmax_status.restype = ci
         L.matmul_forward_argmax_workspace.argtypes = [ci, ci, ci]
@@ -251,6 +256,13 @@ def matmul_forward_argmax(ids, inp, weight, bias, B, T, C, OC, workspace=None):
            "matmul_forward_argmax")
 
 
+def set_stream(stream) -> None:
+    """Make every launcher of this thread use `stream` (a torch.cuda.Stream, a raw
+    hipStream_t value, or None for the null stream)."""
+    raw = getattr(stream, "cuda_stream", stream)
+    lib().gpt2hip_set_stream(raw or None)
+
+
 def read_checkpoint_config(path) -> dict:
     """Header of an llm.c checkpoint file as GPT2(**config) keywords (no GPU needed)."""
     cfg = GPT2Config()
@@ -332,6 +344,13 @@ class GPT2:
             _check(lib().gpt2_forward_status(self._h, a.ctypes.data, B, T), "gpt2_forward")
         else:
             _check(lib().gpt2_forward_device_status(self._h, _i32(inputs), B, T), "gpt2_forward")
+        self._shape = (B, T)
+
+    def forward_graph(self, inputs_device):
+        """forward() of device ids, replayed from a HIP graph captured on first use per (B,T)."""
+        B, T = inputs_device.shape
+        _check(lib().gpt2_forward_graph_status(self._h, _i32(inputs_device), B, T),
+               "gpt2_forward_graph")
         self._shape = (B, T)
 
     def forward_argmax(self, inputs_device):

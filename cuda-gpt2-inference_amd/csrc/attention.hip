@@ -407,14 +407,14 @@ int attention_forward_status(float* out, float* qkvr, float* att, const float* i
     const long long blocks = (long long)nqt * B * NH;
     if (blocks > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "attention_forward: grid too large");
     const float scale_log2e = (1.0f / sqrtf((float)hs)) * 1.4426950408889634f;
-    hipLaunchKernelGGL(attention_flash_kernel, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, 0, out,
+    hipLaunchKernelGGL(attention_flash_kernel, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out,
                        inp, T, NH, nqt, scale_log2e);
   } else {
     if (hs > 256) return fail(GPT2HIP_EINVAL, "attention_forward: head size %d > 256", hs);
     const long long waves = (long long)B * NH * T;
     const long long blocks = (waves + 3) / 4;
     if (blocks > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "attention_forward: grid too large");
-    hipLaunchKernelGGL(attention_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, 0, out, inp,
+    hipLaunchKernelGGL(attention_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), out, inp,
                        B, T, NH, hs, 1.0f / sqrtf((float)hs));
   }
   G2_LAUNCH_CHECK("attention_forward");

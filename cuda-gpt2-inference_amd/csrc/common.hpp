@@ -13,7 +13,12 @@
 namespace g2 {
 
 // ---- host-side error plumbing --------------------------------------------
-char* last_error_buffer();  // thread-local, 512 bytes (defined in capi.hip)
+char* last_error_buffer();  // thread-local, 512 bytes (defined in gpt2.hip)
+
+// The stream every launcher of the calling thread uses (gpt2hip_set_stream); the null
+// stream until set.  Defined in gpt2.hip.
+hipStream_t& stream_slot();
+inline hipStream_t stream() { return stream_slot(); }
 
 inline int fail(int code, const char* fmt, ...) {
   va_list ap;

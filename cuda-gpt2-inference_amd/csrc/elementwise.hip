@@ -101,7 +101,7 @@ static int launch_map(const char* name, float* out, const float* inp1, const flo
     if (n4) {
       const size_t per_block = (size_t)kBlock * kUnroll;
       const unsigned grid = (unsigned)((n4 + per_block - 1) / per_block);
-      hipLaunchKernelGGL((map_vec_kernel<GELU>), dim3(grid), dim3(kBlock), 0, 0,
+      hipLaunchKernelGGL((map_vec_kernel<GELU>), dim3(grid), dim3(kBlock), 0, stream(),
                          reinterpret_cast<f32x4*>(out), reinterpret_cast<const f32x4*>(inp1),
                          reinterpret_cast<const f32x4*>(inp2), n4);
       G2_LAUNCH_CHECK(name);
@@ -110,7 +110,7 @@ static int launch_map(const char* name, float* out, const float* inp1, const flo
   }
   if (done < n) {
     const unsigned grid = (unsigned)((n - done + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL((map_scalar_kernel<GELU>), dim3(grid), dim3(kBlock), 0, 0, out, inp1, inp2,
+    hipLaunchKernelGGL((map_scalar_kernel<GELU>), dim3(grid), dim3(kBlock), 0, stream(), out, inp1, inp2,
                        done, n);
     G2_LAUNCH_CHECK(name);
   }
@@ -171,12 +171,12 @@ int encoder_launch(float* out, const int* inp, const float* wte, const float* wp
   if (C % 4 == 0 && aligned16(out) && aligned16(wte) && aligned16(wpe)) {
     const size_t total4 = total / 4;
     hipLaunchKernelGGL(encoder_vec_kernel, dim3((unsigned)((total4 + kBlock - 1) / kBlock)),
-                       dim3(kBlock), 0, 0, reinterpret_cast<f32x4*>(out), inp,
+                       dim3(kBlock), 0, stream(), reinterpret_cast<f32x4*>(out), inp,
                        reinterpret_cast<const f32x4*>(wte), reinterpret_cast<const f32x4*>(wpe), T,
                        C / 4, total4, V);
   } else {
     hipLaunchKernelGGL(encoder_scalar_kernel, dim3((unsigned)((total + kBlock - 1) / kBlock)),
-                       dim3(kBlock), 0, 0, out, inp, wte, wpe, T, C, total, V);
+                       dim3(kBlock), 0, stream(), out, inp, wte, wpe, T, C, total, V);
   }
   G2_LAUNCH_CHECK("encoder_forward");
   return GPT2HIP_OK;
@@ -217,7 +217,7 @@ int argmax_forward_status(int* ids, const float* logits, int N, int V) {
   if (N < 0 || V < 1) return fail(GPT2HIP_EINVAL, "argmax_forward: bad shape N=%d V=%d", N, V);
   if (N == 0) return GPT2HIP_OK;
   if (!ids || !logits) return fail(GPT2HIP_EINVAL, "argmax_forward: null pointer");
-  hipLaunchKernelGGL(argmax_rows_kernel, dim3(N), dim3(kBlock), 0, 0, ids, logits, V);
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(N), dim3(kBlock), 0, stream(), ids, logits, V);
   G2_LAUNCH_CHECK("argmax_forward");
   return GPT2HIP_OK;
 }

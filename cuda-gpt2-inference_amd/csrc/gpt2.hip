@@ -16,6 +16,11 @@
 
 namespace g2 {
 
+hipStream_t& stream_slot() {
+  static thread_local hipStream_t s = nullptr;
+  return s;
+}
+
 char* last_error_buffer() {
   static thread_local char buf[512] = {0};
   return buf;
@@ -48,11 +53,29 @@ struct GPT2 {
   size_t pairs_bytes;
   int last_B, last_T;
   bool last_has_logits;
+
+  // forward passes captured as HIP graphs, one per (B, T); they hold the activation
+  // pointers, so they are dropped whenever the activations are reallocated
+  struct Captured {
+    int B, T;
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+  };
+  std::vector<Captured> graphs;
 };
 
 namespace g2 {
 
+static void drop_graphs(GPT2* m) {
+  for (auto& g : m->graphs) {
+    (void)hipGraphExecDestroy(g.exec);
+    (void)hipGraphDestroy(g.graph);
+  }
+  m->graphs.clear();
+}
+
 static void free_activations(GPT2* m) {
+  drop_graphs(m);
   void* ptrs[] = {m->ids,  m->res_a, m->res_b, m->ln,     m->qkv,
                   m->atty, m->proj,  m->fch,   m->logits, m->pairs};
   for (void* p : ptrs)
@@ -110,7 +133,7 @@ struct Profile {
     G2_HIP(hipEventCreate(&e));
     events.push_back(e);
     if (cat >= 0) category.push_back(cat);
-    G2_HIP(hipEventRecord(e, 0));
+    G2_HIP(hipEventRecord(e, stream()));
     return GPT2HIP_OK;
   }
   ~Profile() {
@@ -181,6 +204,9 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
 extern "C" {
 
 const char* gpt2hip_last_error(void) { return g2::last_error_buffer(); }
+
+void gpt2hip_set_stream(void* hip_stream) { g2::stream_slot() = static_cast<hipStream_t>(hip_stream); }
+void* gpt2hip_get_stream(void) { return g2::stream_slot(); }
 
 GPT2* gpt2_create(const GPT2Config* config) {
   using namespace g2;
@@ -329,7 +355,9 @@ int gpt2_forward_status(GPT2* model, const int* inputs_host, int B, int T) {
     if (inputs_host[i] < 0 || inputs_host[i] >= model->cfg.vocab_size)
       return fail(GPT2HIP_EINVAL, "gpt2_forward: token id %d at position %zu outside [0,%d)",
                   inputs_host[i], i, model->cfg.vocab_size);
-  G2_HIP(hipMemcpy(model->ids, inputs_host, n * sizeof(int), hipMemcpyHostToDevice));
+  // in stream order after the previous pass; the host buffer is free again on return
+  G2_HIP(hipMemcpyAsync(model->ids, inputs_host, n * sizeof(int), hipMemcpyHostToDevice, stream()));
+  G2_HIP(hipStreamSynchronize(stream()));
   return forward_resident(model, B, T);
 }
 
@@ -342,8 +370,60 @@ int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int
   if (int rc = reserve(model, B, T)) return rc;
   if (!inputs_device) return fail(GPT2HIP_EINVAL, "gpt2_forward_device: null inputs");
   G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
-                        hipMemcpyDeviceToDevice, 0));
+                        hipMemcpyDeviceToDevice, stream()));
   return forward_resident(model, B, T);
+}
+
+int gpt2_forward_graph_status(GPT2* model, const int* inputs_device, int B, int T) {
+  using namespace g2;
+  if (int rc = reserve(model, B, T)) return rc;  // drops the captured graphs if it reallocates
+  if (!inputs_device) return fail(GPT2HIP_EINVAL, "gpt2_forward_graph: null inputs");
+  GPT2::Captured* hit = nullptr;
+  for (auto& g : model->graphs)
+    if (g.B == B && g.T == T) hit = &g;
+  if (!hit) {
+    // One eager pass first: it raises the kernels' LDS limits, which is not stream work
+    // and stays out of the capture.  Then the same launches are recorded from a stream
+    // of their own (default priority) and instantiated.
+    G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
+                          hipMemcpyDeviceToDevice, stream()));
+    if (int rc = forward_resident(model, B, T)) return rc;
+    G2_HIP(hipStreamSynchronize(stream()));
+    hipStream_t cap = nullptr;
+    G2_HIP(hipStreamCreateWithFlags(&cap, hipStreamNonBlocking));
+    hipStream_t const caller = stream_slot();
+    stream_slot() = cap;
+    hipError_t e = hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal);
+    int rc = GPT2HIP_OK;
+    hipGraph_t graph = nullptr;
+    if (e == hipSuccess) {
+      rc = forward_resident(model, B, T);
+      e = hipStreamEndCapture(cap, &graph);  // also ends a capture that a failed launch broke
+    }
+    stream_slot() = caller;
+    (void)hipStreamDestroy(cap);
+    if (rc) {
+      if (graph) (void)hipGraphDestroy(graph);
+      return rc;
+    }
+    if (e != hipSuccess || !graph)
+      return fail(GPT2HIP_EHIP, "gpt2_forward_graph: capture failed: %s", hipGetErrorString(e));
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+      (void)hipGraphDestroy(graph);
+      return fail(GPT2HIP_EHIP, "gpt2_forward_graph: hipGraphInstantiate: %s", hipGetErrorString(e));
+    }
+    model->graphs.push_back({B, T, graph, exec});
+    hit = &model->graphs.back();
+  }
+  G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
+                        hipMemcpyDeviceToDevice, stream()));
+  G2_HIP(hipGraphLaunch(hit->exec, stream()));
+  model->last_B = B;
+  model->last_T = T;
+  model->last_has_logits = true;
+  return GPT2HIP_OK;
 }
 
 int gpt2_forward_argmax_status(GPT2* model, const int* inputs_device, int B, int T,
@@ -353,7 +433,7 @@ int gpt2_forward_argmax_status(GPT2* model, const int* inputs_device, int B, int
   if (!inputs_device || !next_ids_device)
     return fail(GPT2HIP_EINVAL, "gpt2_forward_argmax: null pointer");
   G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
-                        hipMemcpyDeviceToDevice, 0));
+                        hipMemcpyDeviceToDevice, stream()));
   return forward_resident(model, B, T, nullptr, next_ids_device);
 }
 
@@ -364,7 +444,7 @@ int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, i
   if (!inputs_device || !ms_per_category)
     return fail(GPT2HIP_EINVAL, "gpt2_forward_profiled: null pointer");
   G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
-                        hipMemcpyDeviceToDevice, 0));
+                        hipMemcpyDeviceToDevice, stream()));
   Profile prof;
   if (int rc = forward_resident(model, B, T, &prof)) return rc;
   G2_HIP(hipEventSynchronize(prof.events.back()));
@@ -412,14 +492,14 @@ void gpt2hip_timer_destroy(GPT2Timer* t) {
 
 int gpt2hip_timer_start(GPT2Timer* t) {
   if (!t) return g2::fail(GPT2HIP_EINVAL, "gpt2hip_timer_start: null timer");
-  G2_HIP(hipEventRecord(t->start, 0));
+  G2_HIP(hipEventRecord(t->start, g2::stream()));
   return GPT2HIP_OK;
 }
 
 float gpt2hip_timer_stop_ms(GPT2Timer* t) {
   if (!t) return -1.f;
   float ms = -1.f;
-  if (hipEventRecord(t->stop, 0) != hipSuccess || hipEventSynchronize(t->stop) != hipSuccess ||
+  if (hipEventRecord(t->stop, g2::stream()) != hipSuccess || hipEventSynchronize(t->stop) != hipSuccess ||
       hipEventElapsedTime(&ms, t->start, t->stop) != hipSuccess) {
     g2::fail(GPT2HIP_EHIP, "gpt2hip_timer_stop_ms: event timing failed");
     return -1.f;

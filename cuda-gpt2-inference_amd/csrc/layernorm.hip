@@ -156,7 +156,7 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   const bool wide = N >= 4096;
 #define G2_LN(NV, ROWS, EXACT)                                                                  \
   hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED, EXACT>),                           \
-                     dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, 0, \
+                     dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, stream(), \
                      res_out, out, mean, rstd, inp1, inp2, weight, bias, N, C)
 #define G2_LN_ROWS(NV)                         \
   if (wide && C == 256 * NV && N % 4 == 0) {   \
@@ -168,7 +168,7 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   }
   if (!vec) {
     hipLaunchKernelGGL((layernorm_rows_generic_kernel<FUSED>),
-                       dim3((N + kRowsPerBlock - 1) / kRowsPerBlock), block, 0, 0, res_out, out,
+                       dim3((N + kRowsPerBlock - 1) / kRowsPerBlock), block, 0, stream(), res_out, out,
                        mean, rstd, inp1, inp2, weight, bias, N, C);
   } else if (C <= 256) {
     G2_LN_ROWS(1)

@@ -902,7 +902,7 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
                    : (gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true, false>
                            : matmul_mfma_kernel<BM, BN, WGM, WGN, false, false>);
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
                      K, N, ntm, ntn);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
@@ -921,7 +921,7 @@ static int launch_dma(float* out, const float* inp, const float* weight, const f
                    : gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true>
                           : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
                      K, N, ntm, ntn, probe, (int*)nullptr);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
@@ -938,10 +938,10 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
   auto kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, false, true>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)(ntm * ntn)), dim3(NT), lds_bytes, 0, pair_val, inp, weight,
+  hipLaunchKernelGGL(kfn, dim3((unsigned)(ntm * ntn)), dim3(NT), lds_bytes, stream(), pair_val, inp, weight,
                      bias, M, K, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx);
   G2_LAUNCH_CHECK("matmul_forward_argmax");
-  hipLaunchKernelGGL(argmax_pairs_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, 0, ids,
+  hipLaunchKernelGGL(argmax_pairs_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, stream(), ids,
                      pair_val, pair_idx, M, ntn * WGN);
   G2_LAUNCH_CHECK("matmul_forward_argmax");
   return GPT2HIP_OK;
@@ -959,7 +959,7 @@ static int launch_ring(float* out, const float* inp, const float* weight, const 
   auto kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true>
                   : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, 0, out, inp, weight, bias, M,
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
                      K, N, ntm, ntn);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
@@ -978,7 +978,7 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
   if (C % 4 != 0 || !aligned16(inp) || !aligned16(weight)) {
     if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs the MFMA path");
     const size_t total = (size_t)M * OC;
-    hipLaunchKernelGGL(matmul_generic_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, 0,
+    hipLaunchKernelGGL(matmul_generic_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream(),
                        out, inp, weight, bias, M, C, OC, gelu ? 1 : 0);
     G2_LAUNCH_CHECK("matmul_forward");
     return GPT2HIP_OK;
@@ -1079,7 +1079,7 @@ int matmul_forward_argmax_status(int* ids, void* workspace, size_t workspace_byt
   if (!ids || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: null pointer");
   if (C % BK != 0 || !aligned16(inp) || !aligned16(weight) ||
       (long long)C * 192 * 4 >= (1LL << 31)) {
-    hipLaunchKernelGGL(matmul_argmax_generic_kernel, dim3((unsigned)M), dim3(256), 0, 0, ids, inp,
+    hipLaunchKernelGGL(matmul_argmax_generic_kernel, dim3((unsigned)M), dim3(256), 0, stream(), ids, inp,
                        weight, bias, C, OC);
     G2_LAUNCH_CHECK("matmul_forward_argmax");
     return GPT2HIP_OK;

@@ -181,6 +181,13 @@ int gpt2_reserve(GPT2* model, int B, int T);
 int gpt2_forward_status(GPT2* model, const int* inputs_host, int B, int T);
 void gpt2_forward(GPT2* model, const int* inputs_host, int B, int T);
 int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int T);
+/* gpt2_forward_device replayed from a HIP graph: the first call for a (B, T) runs the pass
+ * once eagerly, captures its launches and instantiates the graph; later calls copy the
+ * ids in and launch the graph on the calling thread's stream.  The graphs are dropped
+ * when a larger B*T makes the model reallocate its activations.  No counterpart in the
+ * reference.  (At B=8, T=1024 the launches are not the bound and the graph gains nothing;
+ * it is for short prompts, where the host would otherwise issue ~90 launches per ms.) */
+int gpt2_forward_graph_status(GPT2* model, const int* inputs_device, int B, int T);
 /* Forward pass that keeps only the argmax of every position's logits (greedy next
  * token ids, B*T ints on the device): the lm-head runs as matmul_forward_argmax, the
  * logits buffer is not written and gpt2_argmax_status is unavailable afterwards. */
@@ -210,7 +217,13 @@ const float* gpt2_lnf(const GPT2* model);
 /* Per-position argmax of the last forward's logits into ids_device (B*T). */
 int gpt2_argmax_status(GPT2* model, int* ids_device);
 
-/* Event timer on the null stream (the stream every launcher uses). */
+/* The HIP stream (a hipStream_t) that every launcher, copy and timer of the calling
+ * thread uses from now on; NULL, the initial value, is the null stream.  llm.c launches
+ * on the null stream throughout (train_gpt2_fp32.cu), which is therefore the default. */
+void gpt2hip_set_stream(void* hip_stream);
+void* gpt2hip_get_stream(void);
+
+/* Event timer on the calling thread's stream (the stream its launchers use). */
 typedef struct GPT2Timer GPT2Timer;
 GPT2Timer* gpt2hip_timer_create(void);
 void gpt2hip_timer_destroy(GPT2Timer* t);

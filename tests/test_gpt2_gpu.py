@@ -143,6 +143,63 @@ def test_gpt2_device_ids_outside_vocabulary_give_nan_rows_not_faults():
         model.close()
 
 
+def test_gpt2_graph_replays_match_eager_with_eager_work_between():
+    cfg = dict(max_seq_len=64, vocab_size=211, num_layers=2, num_heads=2, channels=128)
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(syn.make_params(51, perturb_affine=True, **cfg))
+        batches = [torch.from_numpy(syn.make_tokens(60 + i, 2, 48, 211)).cuda() for i in range(4)]
+        other = torch.from_numpy(syn.make_tokens(70, 1, 9, 211)).cuda()
+        eager = []
+        for ids in batches:
+            model.forward(ids)
+            eager.append(model.logits().clone())
+        for rep in range(3):                             # first call captures, the rest replay
+            for ids, want in zip(batches, eager):
+                model.forward_graph(ids)
+                torch.cuda.synchronize()
+                assert torch.equal(model.logits(), want), f"replay {rep}"
+                model.forward(other)                     # eager work between replays
+                scratch = torch.randn(1 << 16, device="cuda").sum().item()
+                assert np.isfinite(scratch)
+        model.forward_graph(other)                       # a second graph, smaller shape
+        model.forward(other)
+        want_other = model.logits().clone()
+        model.forward_graph(other)
+        torch.cuda.synchronize()
+        assert torch.equal(model.logits(), want_other)
+        big = torch.from_numpy(syn.make_tokens(71, 3, 64, 211)).cuda()
+        model.forward_graph(big)                         # reallocation drops the old graphs
+        model.forward_graph(batches[0])                  # and a dropped shape is re-captured
+        torch.cuda.synchronize()
+        assert torch.equal(model.logits(), eager[0])
+    finally:
+        model.close()
+
+
+def test_launchers_follow_the_selected_stream():
+    cfg = dict(max_seq_len=64, vocab_size=211, num_layers=2, num_heads=2, channels=128)
+    model = g2.GPT2(**cfg)
+    side = torch.cuda.Stream()
+    try:
+        model.load_params(syn.make_params(52, **cfg))
+        ids = torch.from_numpy(syn.make_tokens(53, 2, 40, 211)).cuda()
+        model.forward(ids)
+        want = model.logits().clone()
+        torch.cuda.synchronize()
+        g2.set_stream(side)
+        assert g2.lib().gpt2hip_get_stream() == side.cuda_stream
+        model.logits().zero_()
+        torch.cuda.synchronize()
+        model.forward(ids)
+        side.synchronize()                               # waits for the forward only if it ran there
+        assert torch.equal(model.logits(), want)
+    finally:
+        g2.set_stream(None)
+        model.close()
+    assert not g2.lib().gpt2hip_get_stream()
+
+
 def test_gpt2_rejects_bad_inputs():
     model = g2.GPT2(max_seq_len=16, vocab_size=50, num_layers=1, num_heads=1, channels=64)
     try:
