@@ -286,6 +286,39 @@ def clock_probe(g2):
     print(json.dumps({"clock_probe": rows}))
 
 
+def decode_bench(model, cfg, B, T0, steps):
+    """Incremental inference: a prompt of T0 tokens per sequence, then `steps` single-token
+    steps against the key/value cache.  A step is bound by streaming the weights (and the
+    cache rows read by attention) from HBM once."""
+    import torch
+    V, C, L = cfg["vocab_size"], cfg["channels"], cfg["num_layers"]
+    ids = torch.randint(0, V, (B, T0), dtype=torch.int32, device="cuda")
+    nxt = torch.randint(0, V, (steps + 4, B), dtype=torch.int32, device="cuda")
+    model.prefill(ids)
+    for i in range(4):
+        model.decode(nxt[i])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.prefill(ids)
+    torch.cuda.synchronize()
+    prefill_ms = (time.perf_counter() - t0) * 1e3
+    t0 = time.perf_counter()
+    for i in range(steps):
+        model.decode(nxt[4 + i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    pos = T0 + steps / 2
+    weight_bytes = 4 * (L * (12 * C * C + 13 * C) + V * C + 2 * C)
+    cache_bytes = 2 * L * B * pos * C * 4
+    gbs = (weight_bytes + cache_bytes) / ms / 1e6
+    row = {"decode": f"B={B}, prompt T0={T0}, {steps} steps", "prefill_ms": prefill_ms,
+           "ms_per_step": ms, "tokens_per_s": B / ms * 1e3,
+           "bytes_per_step": weight_bytes + cache_bytes, "GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
+           "finite": bool(torch.isfinite(model.step_logits()).all())}
+    log("  decode", json.dumps(row))
+    return row
+
+
 def cpu_baseline(model, cfg, B, T):
     """The CPU oracle on the host cores: one forward of the whole benchmark batch
     (a few seconds on 16 cores), after one untimed pass at B=1 to warm the threads."""
@@ -314,6 +347,8 @@ def main():
     ap.add_argument("--seq-len", type=int, default=1024)
     ap.add_argument("--no-standalone", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--decode", type=int, default=0, metavar="STEPS",
+                    help="time prefill + STEPS single-token decode steps (key/value cache) instead")
     ap.add_argument("--graph", action="store_true",
                     help="also time the forward pass replayed from a HIP graph")
     ap.add_argument("--clock-probe", action="store_true",
@@ -348,6 +383,9 @@ def main():
     init_params_on_device(model, syn, cfg, seed=1337)
     ids = torch.randint(0, cfg["vocab_size"], (B, T), dtype=torch.int32, device="cuda")
     model.reserve(B, T)
+    if args.decode:
+        print(json.dumps({"decode": [decode_bench(model, cfg, B, T, args.decode)]}))
+        return
 
     for _ in range(args.warmup):
         model.forward(ids)

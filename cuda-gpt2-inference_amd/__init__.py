@@ -46,6 +46,7 @@ EXPORTS = (
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
     "gpt2_forward_device_status", "gpt2_forward_graph_status",
+    "gpt2_prefill_status", "gpt2_decode_status", "gpt2_step_logits", "gpt2_cache_length",
     "gpt2_forward_argmax_status",
     "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
@@ -127,6 +128,10 @@ def lib() -> ctypes.CDLL:
         L.gpt2_forward_status.argtypes, L.gpt2_forward_status.restype = [vp, vp, ci, ci], ci
         L.gpt2_forward_device_status.argtypes = [vp, vp, ci, ci]
         L.gpt2_forward_device_status.restype = ci
+        L.gpt2_prefill_status.argtypes, L.gpt2_prefill_status.restype = [vp, vp, ci, ci], ci
+        L.gpt2_decode_status.argtypes, L.gpt2_decode_status.restype = [vp, vp], ci
+        L.gpt2_step_logits.argtypes, L.gpt2_step_logits.restype = [vp], vp
+        L.gpt2_cache_length.argtypes, L.gpt2_cache_length.restype = [vp], ci
         L.gpt2_forward_graph_status.argtypes = [vp, vp, ci, ci]
         L.gpt2_forward_graph_status.restype = ci
         L.gpt2hip_set_stream.argtypes, L.gpt2hip_set_stream.restype = [vp], None
@@ -345,6 +350,28 @@ class GPT2:
         else:
             _check(lib().gpt2_forward_device_status(self._h, _i32(inputs), B, T), "gpt2_forward")
         self._shape = (B, T)
+
+    def prefill(self, inputs_device):
+        """Run a prompt (B,T) of device ids, filling the key/value cache; returns the (B,V)
+        logits of the last position (library-owned memory, overwritten by the next step)."""
+        B, T = inputs_device.shape
+        _check(lib().gpt2_prefill_status(self._h, _i32(inputs_device), B, T), "gpt2_prefill")
+        self._step_batch = B
+        return self.step_logits()
+
+    def decode(self, next_ids_device):
+        """Append one token per sequence ((B,) device ids); returns that position's (B,V) logits."""
+        if next_ids_device.numel() != getattr(self, "_step_batch", -1):
+            raise GPT2HipError("decode: expected one token id per prefilled sequence")
+        _check(lib().gpt2_decode_status(self._h, _i32(next_ids_device)), "gpt2_decode")
+        return self.step_logits()
+
+    def step_logits(self):
+        return _device_view(lib().gpt2_step_logits(self._h),
+                            (self._step_batch, self.config.vocab_size), "float32")
+
+    def cache_length(self) -> int:
+        return lib().gpt2_cache_length(self._h)
 
     def forward_graph(self, inputs_device):
         """forward() of device ids, replayed from a HIP graph captured on first use per (B,T)."""

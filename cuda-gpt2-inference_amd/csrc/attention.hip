@@ -388,6 +388,155 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(float* out, cons
   }
 }
 
+// ---- one new position per sequence against a key/value cache ---------------------
+// Keys and values of past positions live in kc / vc, (B, maxT, C) each, written by
+// kv_store_kernel (a whole prompt) and by this kernel (the new position).  One workgroup
+// of 16 waves per (sequence, head): it appends the new key and value, computes the pos+1
+// scores one wave per position (lanes over the head dimension, DPP reduction), turns them
+// into softmax weights in LDS, and accumulates the weighted values with each wave taking
+// every 16th position; the 16 partial outputs are summed in wave order.  The cache rows
+// are read exactly once: the kernel is bound by that stream of (pos+1) * 2 * hs * 4 bytes.
+constexpr int DEC_WAVES = 16;
+
+__global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode_kernel(
+    float* __restrict__ out, const float* __restrict__ qkv, float* __restrict__ kc,
+    float* __restrict__ vc, int pos, int maxT, int NH, int hs, float scale) {
+  extern __shared__ float dec_lds[];  // scores [pos+1 rounded up to 64] | partial outputs [16][hs]
+  __shared__ float red[2 * DEC_WAVES];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x / NH, head = blockIdx.x % NH;
+  const int C = NH * hs;
+  float* const sc = dec_lds;
+  float* const part = dec_lds + ((pos + 64) & ~63);
+  const float* qrow = qkv + (size_t)b * 3 * C + head * hs;
+  float* const kb = kc + (size_t)b * maxT * C + head * hs;
+  float* const vb = vc + (size_t)b * maxT * C + head * hs;
+
+  for (int d = tid; d < hs; d += DEC_WAVES * kWave) {
+    kb[(size_t)pos * C + d] = qrow[C + d];
+    vb[(size_t)pos * C + d] = qrow[2 * C + d];
+  }
+  float qv[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) qv[j] = (lane + 64 * j < hs) ? qrow[lane + 64 * j] : 0.f;
+  __syncthreads();  // the appended row is visible to the whole workgroup
+
+  // scores
+  float mx = -INFINITY;
+  for (int t0 = wave; t0 <= pos; t0 += 4 * DEC_WAVES) {
+    float p[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int t = min(t0 + u * DEC_WAVES, pos);
+      const float* kr = kb + (size_t)t * C;
+      p[u] = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (lane + 64 * j < hs) p[u] += qv[j] * kr[lane + 64 * j];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int t = t0 + u * DEC_WAVES;
+      const float s = wave_sum(p[u]) * scale;
+      if (t <= pos) {
+        if (lane == 0) sc[t] = s;
+        mx = fmaxf(mx, s);
+      }
+    }
+  }
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  float m = red[0];
+#pragma unroll
+  for (int w = 1; w < DEC_WAVES; w++) m = fmaxf(m, red[w]);  // finite: position 0 always exists
+
+  // softmax weights (unnormalised) and their sum
+  float sum = 0.f;
+  for (int t = tid; t <= pos; t += DEC_WAVES * kWave) {
+    const float e = expf(sc[t] - m);
+    sc[t] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) red[DEC_WAVES + wave] = sum;
+  __syncthreads();
+  float l = 0.f;
+#pragma unroll
+  for (int w = 0; w < DEC_WAVES; w++) l += red[DEC_WAVES + w];
+
+  // weighted values: wave w takes positions w, w + 16, ...
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = wave; t0 <= pos; t0 += 4 * DEC_WAVES) {
+    float vv[4][4], pw[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const int t = t0 + u * DEC_WAVES;
+      pw[u] = (t <= pos) ? sc[t] : 0.f;
+      const float* vr = vb + (size_t)min(t, pos) * C;
+#pragma unroll
+      for (int j = 0; j < 4; j++) vv[u][j] = (lane + 64 * j < hs) ? vr[lane + 64 * j] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[j] += pw[u] * vv[u][j];
+  }
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    if (lane + 64 * j < hs) part[wave * hs + lane + 64 * j] = acc[j];
+  __syncthreads();
+  for (int d = tid; d < hs; d += DEC_WAVES * kWave) {
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; w++) o += part[w * hs + d];
+    out[(size_t)b * C + head * hs + d] = o / l;
+  }
+}
+
+// Copies the key and value thirds of a prompt's packed qkv (B, T, 3C) into the cache
+// (B, maxT, C each) at positions 0..T-1.
+__global__ __launch_bounds__(256) void kv_store_kernel(float* __restrict__ kc, float* __restrict__ vc,
+                                                        const float* __restrict__ qkv, int T,
+                                                        int maxT, int C, size_t total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const size_t bt = i / C;
+  const int c = (int)(i - bt * C);
+  const size_t b = bt / T, t = bt - b * T;
+  const float* src = qkv + bt * 3 * C + C + c;
+  const size_t dst = (b * maxT + t) * C + c;
+  kc[dst] = src[0];
+  vc[dst] = src[C];
+}
+
+int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, int B, int pos,
+                            int maxT, int C, int NH) {
+  if (B < 1 || C < 1 || NH < 1 || C % NH != 0 || pos < 0 || pos >= maxT)
+    return fail(GPT2HIP_EINVAL, "attention_decode: bad shape B=%d C=%d NH=%d pos=%d maxT=%d", B, C,
+                NH, pos, maxT);
+  if (!out || !qkv || !kc || !vc) return fail(GPT2HIP_EINVAL, "attention_decode: null pointer");
+  const int hs = C / NH;
+  if (hs > 256) return fail(GPT2HIP_EINVAL, "attention_decode: head size %d > 256", hs);
+  const size_t lds = ((size_t)((pos + 64) & ~63) + (size_t)DEC_WAVES * hs) * sizeof(float);
+  if (lds > 60 * 1024)
+    return fail(GPT2HIP_EINVAL, "attention_decode: position %d needs %zu bytes of LDS", pos, lds);
+  hipLaunchKernelGGL(attention_decode_kernel, dim3((unsigned)(B * NH)), dim3(DEC_WAVES * kWave), lds,
+                     stream(), out, qkv, kc, vc, pos, maxT, NH, hs, 1.0f / sqrtf((float)hs));
+  G2_LAUNCH_CHECK("attention_decode");
+  return GPT2HIP_OK;
+}
+
+int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C) {
+  const size_t total = (size_t)B * T * C;
+  if (total == 0) return GPT2HIP_OK;
+  hipLaunchKernelGGL(kv_store_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream(), kc,
+                     vc, qkv, T, maxT, C, total);
+  G2_LAUNCH_CHECK("kv_store");
+  return GPT2HIP_OK;
+}
+
 }  // namespace g2
 
 extern "C" {

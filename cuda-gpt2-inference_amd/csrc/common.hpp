@@ -110,6 +110,13 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 }
 #endif
 
+// Decode-step attention of one new position per sequence against the key/value cache
+// (kc, vc: (B, maxT, C)); appends the new key/value at `pos`.  qkv is (B, 3C).
+int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, int B, int pos,
+                            int maxT, int C, int NH);
+// Copies a prompt's keys and values from packed qkv (B, T, 3C) into the cache.
+int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C);
+
 // encoder_forward with an optional on-device check of the token ids against the
 // vocabulary size V (V = 0: ids are trusted, as the reference trusts them).
 int encoder_launch(float* out, const int* inp, const float* wte, const float* wpe, int B, int T,

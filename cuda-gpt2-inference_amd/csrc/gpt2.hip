@@ -54,6 +54,13 @@ struct GPT2 {
   int last_B, last_T;
   bool last_has_logits;
 
+  // key/value cache of the incremental (prefill + decode) path: (L, 2, kv_batch, maxT, C),
+  // and the logits of the newest position, (kv_batch, V)
+  float* kv;
+  float* step_logits;
+  int kv_batch;  // sequences the cache is allocated for
+  int kv_len;    // positions filled so far (the same for every sequence); 0 = empty
+
   // forward passes captured as HIP graphs, one per (B, T); they hold the activation
   // pointers, so they are dropped whenever the activations are reallocated
   struct Captured {
@@ -85,6 +92,30 @@ static void free_activations(GPT2* m) {
   m->pairs = nullptr;
   m->pairs_bytes = 0;
   m->cap_tokens = 0;
+}
+
+static void free_cache(GPT2* m) {
+  if (m->kv) (void)hipFree(m->kv);
+  if (m->step_logits) (void)hipFree(m->step_logits);
+  m->kv = m->step_logits = nullptr;
+  m->kv_batch = m->kv_len = 0;
+}
+
+// Key/value cache and step logits for B sequences of up to max_seq_len positions.
+static int reserve_cache(GPT2* m, int B) {
+  if (B <= m->kv_batch) return GPT2HIP_OK;
+  free_cache(m);
+  const GPT2Config& c = m->cfg;
+  const size_t kv_bytes = (size_t)c.num_layers * 2 * B * c.max_seq_len * c.channels * sizeof(float);
+  hipError_t e = hipMalloc((void**)&m->kv, kv_bytes);
+  if (e == hipSuccess) e = hipMalloc((void**)&m->step_logits, (size_t)B * c.vocab_size * sizeof(float));
+  if (e != hipSuccess) {
+    free_cache(m);
+    return fail(GPT2HIP_ENOMEM, "gpt2: key/value cache for %d sequences (%zu bytes): %s", B, kv_bytes,
+                hipGetErrorString(e));
+  }
+  m->kv_batch = B;
+  return GPT2HIP_OK;
 }
 
 static int check_shape(const GPT2* m, int B, int T) {
@@ -142,9 +173,12 @@ struct Profile {
 };
 
 // The forward pass proper; ids are already in m->ids.  With next_ids the lm-head keeps
-// only the argmax of every row (written there) and m->logits is left untouched.
+// only the argmax of every row (written there) and m->logits is left untouched.  With
+// fill_cache (a prompt: the cache must hold B sequences) every layer's keys and values
+// are also copied into the cache and the lm-head runs on the last position of each
+// sequence only, into m->step_logits.
 static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
-                            int* next_ids = nullptr) {
+                            int* next_ids = nullptr, bool fill_cache = false) {
   const GPT2Config& c = m->cfg;
   const int C = c.channels, L = c.num_layers, NH = c.num_heads, V = c.vocab_size;
   const size_t cs = (size_t)C;
@@ -168,6 +202,11 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
   for (int l = 0; l < L; l++) {
     G2_STEP(GPT2_PROF_MATMUL_QKV, matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
                                  B, T, C, 3 * C));
+    if (fill_cache) {
+      const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
+      G2_TRY(kv_store_launch(m->kv + (2 * (size_t)l) * plane, m->kv + (2 * (size_t)l + 1) * plane, m->qkv,
+                             B, T, c.max_seq_len, C));
+    }
     G2_STEP(GPT2_PROF_ATTENTION, attention_forward_status(m->atty, nullptr, nullptr, m->qkv, B, T, C, NH));
     G2_STEP(GPT2_PROF_MATMUL_ATTPROJ, matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs,
                                  P(P_ATTPROJB) + l * cs, B, T, C, C));
@@ -186,7 +225,12 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
                                                    m->proj, nw, nb, B, T, C));
   }
   // lm-head: weight-tied to wte, no bias, unpadded vocabulary
-  if (next_ids)
+  if (fill_cache) {
+    // rows (b, T-1) of the final layernorm, gathered into the first B rows of m->atty
+    G2_HIP(hipMemcpy2DAsync(m->atty, cs * 4, m->ln + (size_t)(T - 1) * cs, (size_t)T * cs * 4, cs * 4, B,
+                            hipMemcpyDeviceToDevice, stream()));
+    G2_TRY(matmul_forward_status(m->step_logits, m->atty, P(P_WTE), nullptr, B, 1, C, V));
+  } else if (next_ids)
     G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_argmax_status(next_ids, m->pairs, m->pairs_bytes, m->ln,
                                                                   P(P_WTE), nullptr, B, T, C, V));
   else
@@ -195,7 +239,7 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
 #undef G2_TRY
   m->last_B = B;
   m->last_T = T;
-  m->last_has_logits = next_ids == nullptr;
+  m->last_has_logits = next_ids == nullptr && !fill_cache;
   return GPT2HIP_OK;
 }
 
@@ -241,6 +285,7 @@ GPT2* gpt2_create(const GPT2Config* config) {
 void gpt2_destroy(GPT2* model) {
   if (!model) return;
   g2::free_activations(model);
+  g2::free_cache(model);
   if (model->params) (void)hipFree(model->params);
   delete model;
 }
@@ -425,6 +470,75 @@ int gpt2_forward_graph_status(GPT2* model, const int* inputs_device, int B, int 
   model->last_has_logits = true;
   return GPT2HIP_OK;
 }
+
+int gpt2_prefill_status(GPT2* model, const int* inputs_device, int B, int T) {
+  using namespace g2;
+  if (int rc = reserve(model, B, T)) return rc;
+  if (!inputs_device) return fail(GPT2HIP_EINVAL, "gpt2_prefill: null inputs");
+  if (model->kv_batch != B) {  // the cache planes are indexed with the batch it was sized for
+    free_cache(model);
+    if (int rc = reserve_cache(model, B)) return rc;
+  }
+  model->kv_len = 0;
+  G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
+                        hipMemcpyDeviceToDevice, stream()));
+  if (int rc = forward_resident(model, B, T, nullptr, nullptr, true)) return rc;
+  model->kv_len = T;
+  return GPT2HIP_OK;
+}
+
+int gpt2_decode_status(GPT2* model, const int* next_ids_device) {
+  using namespace g2;
+  if (!model || !next_ids_device) return fail(GPT2HIP_EINVAL, "gpt2_decode: null pointer");
+  GPT2* m = model;
+  const GPT2Config& c = m->cfg;
+  if (m->kv_len < 1) return fail(GPT2HIP_EINVAL, "gpt2_decode: no prompt has been prefilled");
+  if (m->kv_len >= c.max_seq_len)
+    return fail(GPT2HIP_EINVAL, "gpt2_decode: the cache is full (%d positions)", c.max_seq_len);
+  const int B = m->kv_batch, pos = m->kv_len;
+  const int C = c.channels, L = c.num_layers, NH = c.num_heads, V = c.vocab_size;
+  const size_t cs = (size_t)C;
+  auto P = [&](int which) { return m->params + m->param_off[which]; };
+#define G2_TRY(call)                  \
+  do {                                \
+    if (int rc_ = (call)) return rc_; \
+  } while (0)
+  // One row per sequence through the same launchers as the full pass; the activation
+  // buffers of the prompt (sized for B*T >= B rows) are reused.
+  float* residual = m->res_a;
+  float* other = m->res_b;
+  G2_HIP(hipMemcpyAsync(m->ids, next_ids_device, (size_t)B * sizeof(int), hipMemcpyDeviceToDevice,
+                        stream()));
+  G2_TRY(encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
+  G2_TRY(layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, 1, C));
+  const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
+  for (int l = 0; l < L; l++) {
+    G2_TRY(matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs, B, 1,
+                                 C, 3 * C));
+    G2_TRY(attention_decode_launch(m->atty, m->qkv, m->kv + (2 * (size_t)l) * plane,
+                                   m->kv + (2 * (size_t)l + 1) * plane, B, pos, c.max_seq_len, C, NH));
+    G2_TRY(matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs, P(P_ATTPROJB) + l * cs, B,
+                                 1, C, C));
+    G2_TRY(fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual, m->proj,
+                                                   P(P_LN2W) + l * cs, P(P_LN2B) + l * cs, B, 1, C));
+    G2_TRY(matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs, P(P_FCB) + l * 4 * cs, B,
+                                      1, C, 4 * C, 1));
+    G2_TRY(matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs, P(P_FCPROJB) + l * cs,
+                                 B, 1, 4 * C, C));
+    const float* nw = (l + 1 < L) ? P(P_LN1W) + (l + 1) * cs : P(P_LNFW);
+    const float* nb = (l + 1 < L) ? P(P_LN1B) + (l + 1) * cs : P(P_LNFB);
+    G2_TRY(fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other, m->proj, nw,
+                                                   nb, B, 1, C));
+  }
+  G2_TRY(matmul_forward_status(m->step_logits, m->ln, P(P_WTE), nullptr, B, 1, C, V));
+#undef G2_TRY
+  m->kv_len = pos + 1;
+  m->last_has_logits = false;  // the (B,T,V) buffer and the activations no longer describe a full pass
+  return GPT2HIP_OK;
+}
+
+const float* gpt2_step_logits(const GPT2* model) { return model ? model->step_logits : nullptr; }
+int gpt2_cache_length(const GPT2* model) { return model ? model->kv_len : 0; }
 
 int gpt2_forward_argmax_status(GPT2* model, const int* inputs_device, int B, int T,
                                int* next_ids_device) {

@@ -2,11 +2,13 @@
 // optional tanh-GELU epilogue.  True fp32 on the matrix cores
 // (v_mfma_f32_32x32x2_f32; gfx950 has no xf32 path).
 //
-// Four kernels share one tiling, LDS layout and MFMA mapping:
+// The kernels (the first three share one tiling, LDS layout and MFMA mapping):
 //   matmul_dma_kernel      K % 32 == 0 (every GPT-2 shape): K slabs go from global
 //                          memory straight into LDS (global_load_lds_dwordx4)
 //   matmul_ring_kernel     the same for problems of few small tiles (short prompts):
 //                          deeper slab ring, optional K split between a tile's waves
+//   matmul_skinny_kernel   at most 16 rows (a decode step): weights streamed through
+//                          registers once, 16x16x4 MFMA, K split over 16 waves
 //   matmul_mfma_kernel     any K % 4 == 0: slabs staged through registers, K tail
 //                          zero-filled
 //   matmul_generic_kernel  anything else (K % 4 != 0, unaligned pointers)
@@ -792,6 +794,103 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
   }
 }
 
+// M <= 16 rows (one token per sequence: a decode step).  Such a product is bound by
+// streaming the weights from HBM once, not by arithmetic, and the problem is small: what
+// matters is that all of it is in flight at once.  A workgroup owns 16 weight rows
+// (output columns) and its 16 waves split K in units of 16 floats; every lane loads its
+// units' 16-byte pieces of the weight row straight into registers (no LDS staging: nothing
+// is reused) and the matching pieces of the activation row, which stay cache-resident, and
+// feeds them to v_mfma_f32_16x16x4_f32 with the same k permutation as the large kernels
+// (element e of a lane's chunk goes to the e-th of four MFMAs).  A = 16 weight rows,
+// B = up to 16 activation rows; lane l of the result holds D[4*(l/16) + v][l % 16].
+// The 16 partial tiles are summed through LDS in wave order, so results are deterministic.
+// RG: groups of 16 weight rows per workgroup (a wave's activation pieces are then used
+// RG times; 2 for wide outputs such as the lm-head, where re-reading the activations per
+// 16 columns would cost as much cache traffic as the weights).  CHUNK: K units a wave has
+// in flight at once.
+constexpr int SK_WAVES = 16;
+
+template <bool GELU, int RG, int CHUNK>
+__global__ __launch_bounds__(SK_WAVES* kWave) void matmul_skinny_kernel(
+    float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
+    const float* __restrict__ bias, int M, int K, int N) {
+  __shared__ float red[SK_WAVES][RG * 4][kWave];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * (16 * RG);
+  const int r16 = lane & 15, kq = lane >> 4;
+  // rows past the end are clamped: they feed result rows / columns that are not stored
+  const float* wp[RG];
+#pragma unroll
+  for (int g = 0; g < RG; g++)
+    wp[g] = weight + (size_t)min(n0 + 16 * g + r16, N - 1) * K + 4 * kq;
+  const float* xp = inp + (size_t)min(r16, M - 1) * K + 4 * kq;
+  const int units = K / 16;
+  const int per = units / SK_WAVES, rem = units % SK_WAVES;
+  const int u0 = wave * per + min(wave, rem);
+  const int cnt = per + (wave < rem ? 1 : 0);  // wave-uniform
+
+  f32x4 acc[RG];
+#pragma unroll
+  for (int g = 0; g < RG; g++) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < cnt; u += CHUNK) {
+    f32x4 wv[RG][CHUNK], xv[CHUNK];
+#pragma unroll
+    for (int c = 0; c < CHUNK; c++) {
+      if (u + c < cnt) {
+        const size_t k = (size_t)(u0 + u + c) * 16;
+#pragma unroll
+        for (int g = 0; g < RG; g++)
+          wv[g][c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp[g] + k));
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNK; c++)
+      if (u + c < cnt) xv[c] = *reinterpret_cast<const f32x4*>(xp + (size_t)(u0 + u + c) * 16);
+#pragma unroll
+    for (int c = 0; c < CHUNK; c++) {
+      if (u + c < cnt) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+          for (int g = 0; g < RG; g++)
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][c][e], xv[c][e], acc[g], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < RG; g++)
+#pragma unroll
+    for (int v = 0; v < 4; v++) red[wave][g * 4 + v][lane] = acc[g][v];
+  __syncthreads();
+  if (tid < 256 * RG) {
+    const int i = tid % (16 * RG), j = tid / (16 * RG);  // output column n0 + i of row j
+    const int g = i >> 4, i16 = i & 15;
+    const int v = i16 & 3, l = (i16 >> 2) * 16 + j;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < SK_WAVES; w++) sum += red[w][g * 4 + v][l];
+    if (j < M && n0 + i < N) {
+      if (bias != nullptr) sum += bias[n0 + i];
+      out[(size_t)j * N + n0 + i] = GELU ? gelu_tanh(sum) : sum;
+    }
+  }
+}
+
+template <bool GELU>
+static int launch_skinny(float* out, const float* inp, const float* weight, const float* bias, int M,
+                         int K, int N) {
+  if (N >= 4096)
+    hipLaunchKernelGGL((matmul_skinny_kernel<GELU, 2, 6>), dim3((unsigned)((N + 31) / 32)),
+                       dim3(SK_WAVES * kWave), 0, stream(), out, inp, weight, bias, M, K, N);
+  else
+    hipLaunchKernelGGL((matmul_skinny_kernel<GELU, 1, 12>), dim3((unsigned)((N + 15) / 16)),
+                       dim3(SK_WAVES * kWave), 0, stream(), out, inp, weight, bias, M, K, N);
+  G2_LAUNCH_CHECK("matmul_forward");
+  return GPT2HIP_OK;
+}
+
 // Any shape, any alignment; one thread per output.  Only used when K is not a
 // multiple of 4 or an operand is not 16-byte aligned.
 __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const float* inp,
@@ -983,6 +1082,9 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
     G2_LAUNCH_CHECK("matmul_forward");
     return GPT2HIP_OK;
   }
+  if (M <= 16 && C % 16 == 0 && !probe)
+    return gelu ? launch_skinny<true>(out, inp, weight, bias, M, C, OC)
+                : launch_skinny<false>(out, inp, weight, bias, M, C, OC);
   // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
   if (C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31)) {
     // Tile choice.  Measured over M = 64 .. 8192 at the GPT-2 shapes, a launch takes

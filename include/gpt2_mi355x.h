@@ -188,6 +188,21 @@ int gpt2_forward_device_status(GPT2* model, const int* inputs_device, int B, int
  * reference.  (At B=8, T=1024 the launches are not the bound and the graph gains nothing;
  * it is for short prompts, where the host would otherwise issue ~90 launches per ms.) */
 int gpt2_forward_graph_status(GPT2* model, const int* inputs_device, int B, int T);
+/* Incremental inference with a key/value cache (no counterpart in the reference, whose
+ * driver only runs whole sequences).  gpt2_prefill runs a prompt of B sequences of T
+ * tokens (ids on the device), stores every layer's keys and values in a cache sized for
+ * max_seq_len positions, and computes the logits of the LAST position of each sequence
+ * only.  gpt2_decode appends one token per sequence (B ids on the device) at the next
+ * position: one row per sequence goes through the same launchers, attention reads the
+ * cache.  After either call gpt2_step_logits() is (B, vocab_size) on the device and
+ * gpt2_cache_length() the number of positions held; the step's logits equal the logits a
+ * full forward pass over the extended sequences gives at that position (to fp32
+ * rounding).  gpt2_logits() / gpt2_argmax_status() describe full passes only. */
+int gpt2_prefill_status(GPT2* model, const int* inputs_device, int B, int T);
+int gpt2_decode_status(GPT2* model, const int* next_ids_device);
+const float* gpt2_step_logits(const GPT2* model);
+int gpt2_cache_length(const GPT2* model);
+
 /* Forward pass that keeps only the argmax of every position's logits (greedy next
  * token ids, B*T ints on the device): the lm-head runs as matmul_forward_argmax, the
  * logits buffer is not written and gpt2_argmax_status is unavailable afterwards. */

@@ -200,6 +200,59 @@ def test_launchers_follow_the_selected_stream():
     assert not g2.lib().gpt2hip_get_stream()
 
 
+@pytest.mark.parametrize("cfg,B,T0,steps", [
+    (dict(max_seq_len=80, vocab_size=331, num_layers=3, num_heads=2, channels=128), 3, 37, 6),
+    (dict(max_seq_len=32, vocab_size=97, num_layers=2, num_heads=2, channels=64), 2, 1, 5),   # hs=32
+    (dict(g2.GPT2_124M), 2, 100, 4),
+])
+def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
+    """Teacher-forced: after a prompt of T0 tokens, every decode step's logits must be the
+    oracle's full-sequence logits at that position."""
+    print(f"gpt2 decode cfg={cfg} B={B} T0={T0} steps={steps}", flush=True)
+    params = syn.make_params(81, perturb_affine=True, **cfg)
+    ids = syn.make_tokens(82, B, T0 + steps, cfg["vocab_size"])
+    exp_logits, _, _ = oracle.gpt2_forward(params, ids, maxT=cfg["max_seq_len"], V=cfg["vocab_size"],
+                                           L=cfg["num_layers"], NH=cfg["num_heads"],
+                                           C=cfg["channels"], want_lnf=True)
+    dids = torch.from_numpy(ids).cuda()
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(params)
+        got = model.prefill(dids[:, :T0].contiguous()).cpu().numpy()
+        assert model.cache_length() == T0
+        d = np.abs(got - exp_logits[:, T0 - 1]).max()
+        print(f"  prefill: max|dlogits|={d:.3e}", flush=True)
+        assert d <= LOGIT_TOL
+        for s in range(steps):
+            got = model.decode(dids[:, T0 + s].contiguous()).cpu().numpy()
+            d = np.abs(got - exp_logits[:, T0 + s]).max()
+            print(f"  step {s}: max|dlogits|={d:.3e}", flush=True)
+            assert d <= LOGIT_TOL
+            assert np.array_equal(got.argmax(-1), exp_logits[:, T0 + s].argmax(-1))
+        assert model.cache_length() == T0 + steps
+        # a new prompt with another batch size restarts the cache
+        got = model.prefill(dids[:1, :T0].contiguous()).cpu().numpy()
+        assert np.abs(got - exp_logits[:1, T0 - 1]).max() <= LOGIT_TOL
+    finally:
+        model.close()
+
+
+def test_gpt2_decode_error_paths():
+    cfg = dict(max_seq_len=8, vocab_size=50, num_layers=1, num_heads=1, channels=64)
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(syn.make_params(83, **cfg))
+        tok = torch.zeros(2, dtype=torch.int32, device="cuda")
+        assert g2.lib().gpt2_decode_status(model._h, tok.data_ptr()) == 1      # nothing prefilled
+        model.prefill(torch.from_numpy(syn.make_tokens(84, 2, 7, 50)).cuda())
+        model.decode(tok)                                                       # position 7: the last
+        assert model.cache_length() == 8
+        with pytest.raises(g2.GPT2HipError, match="full"):
+            model.decode(tok)
+    finally:
+        model.close()
+
+
 def test_gpt2_rejects_bad_inputs():
     model = g2.GPT2(max_seq_len=16, vocab_size=50, num_layers=1, num_heads=1, channels=64)
     try:

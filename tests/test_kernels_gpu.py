@@ -217,6 +217,7 @@ def run_matmul(x, w, b, gelu=None):
     (256, 768, 2304), (256, 3072, 768),                                          # B=4, T=64
     (4096, 1024, 3072), (4096, 4096, 1024),                                      # GPT-2 350M
     (4096, 768, 768), (1024, 1024, 1024), (1000, 96, 1000), (64, 768, 3072),     # 64x64 / 32x32 tiles
+    (1, 768, 2304), (8, 3072, 768), (16, 768, 50257), (5, 48, 37), (3, 1040, 100),  # <= 16 rows
     (128, 32, 192), (1, 4, 1), (130, 36, 200), (77, 100, 81), (300, 768, 50),    # edges
 ])
 def test_matmul_bias(M, C, OC):
@@ -249,7 +250,7 @@ def test_matmul_generic_path_unaligned_k():
     assert_close(run_matmul(x, w, None), oracle.matmul_forward(x, w, None), "matmul generic nobias")
 
 
-@pytest.mark.parametrize("M,C,OC", [(8192, 768, 3072), (256, 768, 3072), (70, 64, 100)])
+@pytest.mark.parametrize("M,C,OC", [(8192, 768, 3072), (256, 768, 3072), (70, 64, 100), (8, 768, 3072)])
 def test_matmul_gelu_epilogue(M, C, OC):
     say(f"matmul+gelu M={M} C={C} OC={OC}")
     x, w, b = mm_inputs(M, C, OC, 123)
