@@ -495,6 +495,104 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode_kernel(
   }
 }
 
+// Head size 64 with 16-byte aligned rows: 16 lanes cover one cache row with 128-bit loads,
+// so a wave instruction brings four positions (1 KiB) and a wave keeps DEC_UNROLL of them
+// in flight; position t = 4 * (wave + 16 * i) + lane / 16.
+constexpr int DEC_UNROLL = 8;
+
+__global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
+    float* __restrict__ out, const float* __restrict__ qkv, float* __restrict__ kc,
+    float* __restrict__ vc, int pos, int maxT, int NH, float scale) {
+  extern __shared__ float dec_lds[];  // scores [pos+1 rounded up to 64] | partial outputs [16][64]
+  __shared__ float red[2 * DEC_WAVES];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int p4 = lane >> 4, sub = lane & 15;
+  const int b = blockIdx.x / NH, head = blockIdx.x % NH;
+  const int C = NH * 64;
+  float* const sc = dec_lds;
+  float* const part = dec_lds + ((pos + 64) & ~63);
+  const float* qrow = qkv + (size_t)b * 3 * C + head * 64;
+  float* const kb = kc + (size_t)b * maxT * C + head * 64 + 4 * sub;
+  float* const vb = vc + (size_t)b * maxT * C + head * 64 + 4 * sub;
+
+  if (tid < 16) {
+    *reinterpret_cast<f32x4*>(kb + (size_t)pos * C) = *reinterpret_cast<const f32x4*>(qrow + C + 4 * sub);
+    *reinterpret_cast<f32x4*>(vb + (size_t)pos * C) =
+        *reinterpret_cast<const f32x4*>(qrow + 2 * C + 4 * sub);
+  }
+  const f32x4 q4 = *reinterpret_cast<const f32x4*>(qrow + 4 * sub);
+  __syncthreads();  // the appended row is visible to the whole workgroup
+
+  float mx = -INFINITY;
+  for (int g0 = wave; 4 * g0 <= pos; g0 += DEC_UNROLL * DEC_WAVES) {
+    f32x4 kf[DEC_UNROLL];
+#pragma unroll
+    for (int u = 0; u < DEC_UNROLL; u++) {
+      const int t = min(4 * (g0 + u * DEC_WAVES) + p4, pos);
+      kf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb + (size_t)t * C));
+    }
+#pragma unroll
+    for (int u = 0; u < DEC_UNROLL; u++) {
+      const int t = 4 * (g0 + u * DEC_WAVES) + p4;
+      const f32x4 pr = q4 * kf[u];
+      const float s = row16_sum((pr[0] + pr[1]) + (pr[2] + pr[3])) * scale;
+      if (t <= pos) {
+        if (sub == 0) sc[t] = s;
+        mx = fmaxf(mx, s);
+      }
+    }
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  float m = red[0];
+#pragma unroll
+  for (int w = 1; w < DEC_WAVES; w++) m = fmaxf(m, red[w]);  // finite: position 0 always exists
+
+  float sum = 0.f;
+  for (int t = tid; t <= pos; t += DEC_WAVES * kWave) {
+    const float e = expf(sc[t] - m);
+    sc[t] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) red[DEC_WAVES + wave] = sum;
+  __syncthreads();
+  float l = 0.f;
+#pragma unroll
+  for (int w = 0; w < DEC_WAVES; w++) l += red[DEC_WAVES + w];
+
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int g0 = wave; 4 * g0 <= pos; g0 += DEC_UNROLL * DEC_WAVES) {
+    f32x4 vf[DEC_UNROLL];
+    float pw[DEC_UNROLL];
+#pragma unroll
+    for (int u = 0; u < DEC_UNROLL; u++) {
+      const int t = 4 * (g0 + u * DEC_WAVES) + p4;
+      pw[u] = (t <= pos) ? sc[t] : 0.f;
+      vf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb + (size_t)min(t, pos) * C));
+    }
+#pragma unroll
+    for (int u = 0; u < DEC_UNROLL; u++) acc += pw[u] * vf[u];
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    acc[e] += __shfl_xor(acc[e], 16, 64);
+    acc[e] += __shfl_xor(acc[e], 32, 64);
+  }
+  if (p4 == 0) *reinterpret_cast<f32x4*>(part + wave * 64 + 4 * sub) = acc;
+  __syncthreads();
+  if (tid < 64) {
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; w++) o += part[w * 64 + tid];
+    out[(size_t)b * C + head * 64 + tid] = o / l;
+  }
+}
+
 // Copies the key and value thirds of a prompt's packed qkv (B, T, 3C) into the cache
 // (B, maxT, C each) at positions 0..T-1.
 __global__ __launch_bounds__(256) void kv_store_kernel(float* __restrict__ kc, float* __restrict__ vc,
@@ -522,8 +620,12 @@ int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, 
   const size_t lds = ((size_t)((pos + 64) & ~63) + (size_t)DEC_WAVES * hs) * sizeof(float);
   if (lds > 60 * 1024)
     return fail(GPT2HIP_EINVAL, "attention_decode: position %d needs %zu bytes of LDS", pos, lds);
-  hipLaunchKernelGGL(attention_decode_kernel, dim3((unsigned)(B * NH)), dim3(DEC_WAVES * kWave), lds,
-                     stream(), out, qkv, kc, vc, pos, maxT, NH, hs, 1.0f / sqrtf((float)hs));
+  if (hs == 64 && aligned16(qkv) && aligned16(kc) && aligned16(vc))
+    hipLaunchKernelGGL(attention_decode64_kernel, dim3((unsigned)(B * NH)), dim3(DEC_WAVES * kWave), lds,
+                       stream(), out, qkv, kc, vc, pos, maxT, NH, 1.0f / sqrtf(64.f));
+  else
+    hipLaunchKernelGGL(attention_decode_kernel, dim3((unsigned)(B * NH)), dim3(DEC_WAVES * kWave), lds,
+                       stream(), out, qkv, kc, vc, pos, maxT, NH, hs, 1.0f / sqrtf((float)hs));
   G2_LAUNCH_CHECK("attention_decode");
   return GPT2HIP_OK;
 }

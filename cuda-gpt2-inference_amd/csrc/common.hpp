@@ -78,6 +78,15 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Sum over each row of 16 lanes (all 16 lanes of the row receive it).
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp<0x141>(v);  // row_half_mirror
+  v += dpp<0x140>(v);  // row_mirror
+  return v;
+}
+
 // (value, index) combination of an argmax: the larger value wins, the smaller index
 // among equal values.  NaN never wins (every comparison with it is false).
 // Written with selects: as branches, a chain of these turns into divergent control flow.
@@ -109,6 +118,13 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 #endif
+
+// The <= 16-row GEMM with optional fused input layernorm (ln_w, ln_b: over K) and fused
+// residual add (resid, may alias out): out = resid + act(LN(inp) . weight^T + bias).
+bool skinny_supported(int M, int K, bool ln, const void* inp, const void* weight);
+int skinny_launch(float* out, const float* inp, const float* weight, const float* bias,
+                  const float* ln_w, const float* ln_b, const float* resid, int M, int K, int N,
+                  bool gelu);
 
 // Decode-step attention of one new position per sequence against the key/value cache
 // (kc, vc: (B, maxT, C)); appends the new key/value at `pos`.  qkv is (B, 3C).

@@ -503,34 +503,56 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device) {
   do {                                \
     if (int rc_ = (call)) return rc_; \
   } while (0)
-  // One row per sequence through the same launchers as the full pass; the activation
-  // buffers of the prompt (sized for B*T >= B rows) are reused.
+  // One row per sequence; the activation buffers of the prompt (sized for B*T >= B rows)
+  // are reused.
   float* residual = m->res_a;
   float* other = m->res_b;
   G2_HIP(hipMemcpyAsync(m->ids, next_ids_device, (size_t)B * sizeof(int), hipMemcpyDeviceToDevice,
                         stream()));
   G2_TRY(encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
-  G2_TRY(layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, 1, C));
   const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
-  for (int l = 0; l < L; l++) {
-    G2_TRY(matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs, B, 1,
-                                 C, 3 * C));
-    G2_TRY(attention_decode_launch(m->atty, m->qkv, m->kv + (2 * (size_t)l) * plane,
-                                   m->kv + (2 * (size_t)l + 1) * plane, B, pos, c.max_seq_len, C, NH));
-    G2_TRY(matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs, P(P_ATTPROJB) + l * cs, B,
-                                 1, C, C));
-    G2_TRY(fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual, m->proj,
-                                                   P(P_LN2W) + l * cs, P(P_LN2B) + l * cs, B, 1, C));
-    G2_TRY(matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs, P(P_FCB) + l * 4 * cs, B,
-                                      1, C, 4 * C, 1));
-    G2_TRY(matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs, P(P_FCPROJB) + l * cs,
-                                 B, 1, 4 * C, C));
-    const float* nw = (l + 1 < L) ? P(P_LN1W) + (l + 1) * cs : P(P_LNFW);
-    const float* nb = (l + 1 < L) ? P(P_LN1B) + (l + 1) * cs : P(P_LNFB);
-    G2_TRY(fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other, m->proj, nw,
-                                                   nb, B, 1, C));
+  if (skinny_supported(B, C, true, residual, m->params) && skinny_supported(B, 4 * C, false, m->fch, m->params)) {
+    // Up to 16 sequences: five launches per block.  The layernorms run inside the GEMMs
+    // that consume them and the residual adds inside the GEMMs that produce the update:
+    //   qkv = LN1(x) Wqkv ; attention ; x += atty Wproj ; h = gelu(LN2(x) Wfc) ; x += h Wfcproj
+    float* x = residual;
+    for (int l = 0; l < L; l++) {
+      G2_TRY(skinny_launch(m->qkv, x, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
+                           P(P_LN1W) + l * cs, P(P_LN1B) + l * cs, nullptr, B, C, 3 * C, false));
+      G2_TRY(attention_decode_launch(m->atty, m->qkv, m->kv + (2 * (size_t)l) * plane,
+                                     m->kv + (2 * (size_t)l + 1) * plane, B, pos, c.max_seq_len, C, NH));
+      G2_TRY(skinny_launch(x, m->atty, P(P_ATTPROJW) + l * cs * cs, P(P_ATTPROJB) + l * cs, nullptr,
+                           nullptr, x, B, C, C, false));
+      G2_TRY(skinny_launch(m->fch, x, P(P_FCW) + l * 4 * cs * cs, P(P_FCB) + l * 4 * cs,
+                           P(P_LN2W) + l * cs, P(P_LN2B) + l * cs, nullptr, B, C, 4 * C, true));
+      G2_TRY(skinny_launch(x, m->fch, P(P_FCPROJW) + l * 4 * cs * cs, P(P_FCPROJB) + l * cs, nullptr,
+                           nullptr, x, B, 4 * C, C, false));
+    }
+    G2_TRY(skinny_launch(m->step_logits, x, P(P_WTE), nullptr, P(P_LNFW), P(P_LNFB), nullptr, B, C, V,
+                         false));
+  } else {
+    // More sequences (or sizes the fused kernel does not take): the launchers of the full pass.
+    G2_TRY(layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, 1, C));
+    for (int l = 0; l < L; l++) {
+      G2_TRY(matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs, B,
+                                   1, C, 3 * C));
+      G2_TRY(attention_decode_launch(m->atty, m->qkv, m->kv + (2 * (size_t)l) * plane,
+                                     m->kv + (2 * (size_t)l + 1) * plane, B, pos, c.max_seq_len, C, NH));
+      G2_TRY(matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs, P(P_ATTPROJB) + l * cs,
+                                   B, 1, C, C));
+      G2_TRY(fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual, m->proj,
+                                                     P(P_LN2W) + l * cs, P(P_LN2B) + l * cs, B, 1, C));
+      G2_TRY(matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs, P(P_FCB) + l * 4 * cs,
+                                        B, 1, C, 4 * C, 1));
+      G2_TRY(matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
+                                   P(P_FCPROJB) + l * cs, B, 1, 4 * C, C));
+      const float* nw = (l + 1 < L) ? P(P_LN1W) + (l + 1) * cs : P(P_LNFW);
+      const float* nb = (l + 1 < L) ? P(P_LN1B) + (l + 1) * cs : P(P_LNFB);
+      G2_TRY(fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other, m->proj,
+                                                     nw, nb, B, 1, C));
+    }
+    G2_TRY(matmul_forward_status(m->step_logits, m->ln, P(P_WTE), nullptr, B, 1, C, V));
   }
-  G2_TRY(matmul_forward_status(m->step_logits, m->ln, P(P_WTE), nullptr, B, 1, C, V));
 #undef G2_TRY
   m->kv_len = pos + 1;
   m->last_has_logits = false;  // the (B,T,V) buffer and the activations no longer describe a full pass

@@ -804,89 +804,130 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
 // (element e of a lane's chunk goes to the e-th of four MFMAs).  A = 16 weight rows,
 // B = up to 16 activation rows; lane l of the result holds D[4*(l/16) + v][l % 16].
 // The 16 partial tiles are summed through LDS in wave order, so results are deterministic.
-// RG: groups of 16 weight rows per workgroup (a wave's activation pieces are then used
-// RG times; 2 for wide outputs such as the lm-head, where re-reading the activations per
-// 16 columns would cost as much cache traffic as the weights).  CHUNK: K units a wave has
-// in flight at once.
+// LN: the activation rows are layer-normalised on the way in (mean / variance over K by
+// llm.c's two passes, then gamma and beta), which needs a wave's whole K share in
+// registers at once (K <= 16 * 16 * SK_CHUNK_LN = 1536); every workgroup recomputes the statistics
+// of the <= 16 rows from the pieces its waves hold anyway.  resid: added to the result
+// (out may alias it).  Together these let a decode step run a transformer block in five
+// launches instead of seven.
 constexpr int SK_WAVES = 16;
+// K units (of 16 floats) a wave has in flight at once; fewer with LN, whose statistics
+// and affine terms need registers of their own (16 waves leave 128 per lane)
+constexpr int SK_CHUNK_PLAIN = 12, SK_CHUNK_LN = 6;
 
-template <bool GELU, int RG, int CHUNK>
+template <bool GELU, bool LN>
 __global__ __launch_bounds__(SK_WAVES* kWave) void matmul_skinny_kernel(
-    float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, int M, int K, int N) {
-  __shared__ float red[SK_WAVES][RG * 4][kWave];
+    float* out, const float* __restrict__ inp, const float* __restrict__ weight,
+    const float* __restrict__ bias, const float* __restrict__ ln_w, const float* __restrict__ ln_b,
+    const float* resid, int M, int K, int N) {
+  constexpr int SK_CHUNK = LN ? SK_CHUNK_LN : SK_CHUNK_PLAIN;
+  __shared__ float red[SK_WAVES][4][kWave];
+  __shared__ float stat[2][SK_WAVES][16];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n0 = blockIdx.x * (16 * RG);
+  const int n0 = blockIdx.x * 16;
   const int r16 = lane & 15, kq = lane >> 4;
   // rows past the end are clamped: they feed result rows / columns that are not stored
-  const float* wp[RG];
-#pragma unroll
-  for (int g = 0; g < RG; g++)
-    wp[g] = weight + (size_t)min(n0 + 16 * g + r16, N - 1) * K + 4 * kq;
+  const float* wp = weight + (size_t)min(n0 + r16, N - 1) * K + 4 * kq;
   const float* xp = inp + (size_t)min(r16, M - 1) * K + 4 * kq;
   const int units = K / 16;
   const int per = units / SK_WAVES, rem = units % SK_WAVES;
   const int u0 = wave * per + min(wave, rem);
-  const int cnt = per + (wave < rem ? 1 : 0);  // wave-uniform
+  const int cnt = per + (wave < rem ? 1 : 0);  // wave-uniform; <= SK_CHUNK when LN
 
-  f32x4 acc[RG];
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < cnt || (LN && u == 0); u += SK_CHUNK) {
+    f32x4 wv[SK_CHUNK], xv[SK_CHUNK];
 #pragma unroll
-  for (int g = 0; g < RG; g++) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int u = 0; u < cnt; u += CHUNK) {
-    f32x4 wv[RG][CHUNK], xv[CHUNK];
+    for (int c = 0; c < SK_CHUNK; c++)
+      if (u + c < cnt)
+        wv[c] = __builtin_nontemporal_load(
+            reinterpret_cast<const f32x4*>(wp + (size_t)(u0 + u + c) * 16));
 #pragma unroll
-    for (int c = 0; c < CHUNK; c++) {
-      if (u + c < cnt) {
-        const size_t k = (size_t)(u0 + u + c) * 16;
+    for (int c = 0; c < SK_CHUNK; c++)
+      if (u + c < cnt) xv[c] = *reinterpret_cast<const f32x4*>(xp + (size_t)(u0 + u + c) * 16);
+    if (LN) {
+      // row r16's statistics: lanes r16, r16+16, r16+32, r16+48 of all 16 waves hold the row
+      float s = 0.f;
 #pragma unroll
-        for (int g = 0; g < RG; g++)
-          wv[g][c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp[g] + k));
-      }
+      for (int c = 0; c < SK_CHUNK; c++)
+        if (c < cnt) s += (xv[c][0] + xv[c][1]) + (xv[c][2] + xv[c][3]);
+      s += __shfl_xor(s, 16, 64);
+      s += __shfl_xor(s, 32, 64);
+      if (kq == 0) stat[0][wave][r16] = s;
+      __syncthreads();
+      float mean = 0.f;
+#pragma unroll
+      for (int w = 0; w < SK_WAVES; w++) mean += stat[0][w][r16];
+      mean /= (float)K;
+      float q = 0.f;
+#pragma unroll
+      for (int c = 0; c < SK_CHUNK; c++)
+        if (c < cnt) {
+          const f32x4 d = xv[c] - mean;
+          q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+        }
+      q += __shfl_xor(q, 16, 64);
+      q += __shfl_xor(q, 32, 64);
+      if (kq == 0) stat[1][wave][r16] = q;
+      __syncthreads();
+      float var = 0.f;
+#pragma unroll
+      for (int w = 0; w < SK_WAVES; w++) var += stat[1][w][r16];
+      const float rstd = 1.0f / sqrtf(var / (float)K + 1e-5f);
+#pragma unroll
+      for (int c = 0; c < SK_CHUNK; c++)
+        if (c < cnt) {
+          const size_t k = (size_t)(u0 + c) * 16 + 4 * kq;
+          const f32x4 g = *reinterpret_cast<const f32x4*>(ln_w + k);
+          const f32x4 be = *reinterpret_cast<const f32x4*>(ln_b + k);
+          xv[c] = (xv[c] - mean) * rstd * g + be;
+        }
     }
 #pragma unroll
-    for (int c = 0; c < CHUNK; c++)
-      if (u + c < cnt) xv[c] = *reinterpret_cast<const f32x4*>(xp + (size_t)(u0 + u + c) * 16);
-#pragma unroll
-    for (int c = 0; c < CHUNK; c++) {
+    for (int c = 0; c < SK_CHUNK; c++) {
       if (u + c < cnt) {
 #pragma unroll
         for (int e = 0; e < 4; e++)
-#pragma unroll
-          for (int g = 0; g < RG; g++)
-            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][c][e], xv[c][e], acc[g], 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[c][e], xv[c][e], acc, 0, 0, 0);
       }
     }
   }
 #pragma unroll
-  for (int g = 0; g < RG; g++)
-#pragma unroll
-    for (int v = 0; v < 4; v++) red[wave][g * 4 + v][lane] = acc[g][v];
+  for (int v = 0; v < 4; v++) red[wave][v][lane] = acc[v];
   __syncthreads();
-  if (tid < 256 * RG) {
-    const int i = tid % (16 * RG), j = tid / (16 * RG);  // output column n0 + i of row j
-    const int g = i >> 4, i16 = i & 15;
-    const int v = i16 & 3, l = (i16 >> 2) * 16 + j;
+  if (tid < 256) {
+    const int i = tid & 15, j = tid >> 4;  // output column n0 + i of row j
+    const int v = i & 3, l = (i >> 2) * 16 + j;
     float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < SK_WAVES; w++) sum += red[w][g * 4 + v][l];
+    for (int w = 0; w < SK_WAVES; w++) sum += red[w][v][l];
     if (j < M && n0 + i < N) {
       if (bias != nullptr) sum += bias[n0 + i];
-      out[(size_t)j * N + n0 + i] = GELU ? gelu_tanh(sum) : sum;
+      if (GELU) sum = gelu_tanh(sum);
+      if (resid != nullptr) sum += resid[(size_t)j * N + n0 + i];
+      out[(size_t)j * N + n0 + i] = sum;
     }
   }
 }
 
-template <bool GELU>
-static int launch_skinny(float* out, const float* inp, const float* weight, const float* bias, int M,
-                         int K, int N) {
-  if (N >= 4096)
-    hipLaunchKernelGGL((matmul_skinny_kernel<GELU, 2, 6>), dim3((unsigned)((N + 31) / 32)),
-                       dim3(SK_WAVES * kWave), 0, stream(), out, inp, weight, bias, M, K, N);
-  else
-    hipLaunchKernelGGL((matmul_skinny_kernel<GELU, 1, 12>), dim3((unsigned)((N + 15) / 16)),
-                       dim3(SK_WAVES * kWave), 0, stream(), out, inp, weight, bias, M, K, N);
+// Whether skinny_launch can take the shape (and, with LN, normalise on the way in).
+bool skinny_supported(int M, int K, bool ln, const void* inp, const void* weight) {
+  if (M < 1 || M > 16 || K % 16 != 0 || !aligned16(inp) || !aligned16(weight)) return false;
+  return !ln || (K / 16 + SK_WAVES - 1) / SK_WAVES <= SK_CHUNK_LN;
+}
+
+int skinny_launch(float* out, const float* inp, const float* weight, const float* bias,
+                  const float* ln_w, const float* ln_b, const float* resid, int M, int K, int N,
+                  bool gelu) {
+  const bool ln = ln_w != nullptr;
+  if (!skinny_supported(M, K, ln, inp, weight) || (ln && (!ln_b || !aligned16(ln_w) || !aligned16(ln_b))))
+    return fail(GPT2HIP_EINVAL, "matmul (<= 16 rows): unsupported shape M=%d K=%d", M, K);
+  auto kfn = gelu ? (ln ? matmul_skinny_kernel<true, true> : matmul_skinny_kernel<true, false>)
+                  : (ln ? matmul_skinny_kernel<false, true> : matmul_skinny_kernel<false, false>);
+  hipLaunchKernelGGL(kfn, dim3((unsigned)((N + 15) / 16)), dim3(SK_WAVES * kWave), 0, stream(), out, inp,
+                     weight, bias, ln_w, ln_b, resid, M, K, N);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1083,8 +1124,7 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
     return GPT2HIP_OK;
   }
   if (M <= 16 && C % 16 == 0 && !probe)
-    return gelu ? launch_skinny<true>(out, inp, weight, bias, M, C, OC)
-                : launch_skinny<false>(out, inp, weight, bias, M, C, OC);
+    return skinny_launch(out, inp, weight, bias, nullptr, nullptr, nullptr, M, C, OC, gelu);
   // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
   if (C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31)) {
     // Tile choice.  Measured over M = 64 .. 8192 at the GPT-2 shapes, a launch takes

@@ -204,6 +204,8 @@ def test_launchers_follow_the_selected_stream():
     (dict(max_seq_len=80, vocab_size=331, num_layers=3, num_heads=2, channels=128), 3, 37, 6),
     (dict(max_seq_len=32, vocab_size=97, num_layers=2, num_heads=2, channels=64), 2, 1, 5),   # hs=32
     (dict(g2.GPT2_124M), 2, 100, 4),
+    (dict(max_seq_len=48, vocab_size=211, num_layers=2, num_heads=2, channels=128), 17, 20, 3),  # > 16 rows
+    (dict(max_seq_len=40, vocab_size=97, num_layers=2, num_heads=3, channels=60), 2, 9, 3),      # C % 16 != 0
 ])
 def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
     """Teacher-forced: after a prompt of T0 tokens, every decode step's logits must be the
