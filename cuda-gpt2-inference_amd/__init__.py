@@ -20,7 +20,8 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_HERE)
 LIB_PATH = os.path.join(_HERE, "libgpt2_mi355x.so")
-SOURCES = ("layernorm.hip", "elementwise.hip", "matmul.hip", "attention.hip", "gpt2.hip")
+SOURCES = ("layernorm.hip", "elementwise.hip", "matmul.hip", "attention.hip", "decode.hip",
+           "gpt2.hip")
 HIPCC_FLAGS = (
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
     # packed-fp32 VALU forms are switched off for every HIP translation unit
@@ -46,7 +47,7 @@ EXPORTS = (
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
     "gpt2_forward_device_status", "gpt2_forward_graph_status",
-    "gpt2_prefill_status", "gpt2_decode_status", "gpt2_step_logits", "gpt2_cache_length",
+    "gpt2_prefill_status", "gpt2_decode_status", "gpt2_decode_options", "gpt2_step_logits", "gpt2_cache_length",
     "gpt2_forward_argmax_status",
     "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
@@ -130,6 +131,7 @@ def lib() -> ctypes.CDLL:
         L.gpt2_forward_device_status.restype = ci
         L.gpt2_prefill_status.argtypes, L.gpt2_prefill_status.restype = [vp, vp, ci, ci], ci
         L.gpt2_decode_status.argtypes, L.gpt2_decode_status.restype = [vp, vp], ci
+        L.gpt2_decode_options.argtypes, L.gpt2_decode_options.restype = [vp, ci, ctypes.c_uint], ci
         L.gpt2_step_logits.argtypes, L.gpt2_step_logits.restype = [vp], vp
         L.gpt2_cache_length.argtypes, L.gpt2_cache_length.restype = [vp], ci
         L.gpt2_forward_graph_status.argtypes = [vp, vp, ci, ci]
@@ -365,6 +367,10 @@ class GPT2:
             raise GPT2HipError("decode: expected one token id per prefilled sequence")
         _check(lib().gpt2_decode_status(self._h, _i32(next_ids_device)), "gpt2_decode")
         return self.step_logits()
+
+    def decode_options(self, persistent: bool = True, spin_limit: int = 1 << 21):
+        """Choose between the persistent decode-step kernel and one launch per operation."""
+        _check(lib().gpt2_decode_options(self._h, int(persistent), spin_limit), "gpt2_decode_options")
 
     def step_logits(self):
         return _device_view(lib().gpt2_step_logits(self._h),

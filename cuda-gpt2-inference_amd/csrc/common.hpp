@@ -133,6 +133,27 @@ int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, 
 // Copies a prompt's keys and values from packed qkv (B, T, 3C) into the cache.
 int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C);
 
+// One decode step as a single persistent kernel (decode.hip): every pointer is device memory.
+struct DecodeStep {
+  const float *wte, *wpe_row, *ln1w, *ln1b, *qkvw, *qkvb, *attprojw, *attprojb, *ln2w, *ln2b, *fcw,
+      *fcb, *fcprojw, *fcprojb, *lnfw, *lnfb;
+  const int* ids;      // (B) new token of every sequence
+  float* kv;           // keys of layer l at kv + 2*l*plane, values at kv + (2*l+1)*plane: (B, maxT, C)
+  size_t plane;
+  float *x, *qkv, *atty, *h;  // (B,C) (B,3C) (B,C) (B,4C), handed between workgroups
+  float* logits;              // (B,V)
+  unsigned* flags;            // [gridDim.x * FLAG_STRIDE] epochs, then the error word
+  unsigned epoch0;            // flags hold values below epoch0 + 1 when the kernel starts
+  unsigned spin_limit;
+  int B, C, L, NH, V, pos, maxT;
+};
+// Whether the persistent kernel takes the model at B sequences on this device; the bytes of
+// its flag array (zero-filled by the owner before the first step); the launch itself, which
+// uses barrier epochs step.epoch0 + 1 .. step.epoch0 + 5 * L.
+bool decode_step_supported(const GPT2Config& c, int B, int device);
+size_t decode_step_flag_bytes(int device);
+int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device);
+
 // encoder_forward with an optional on-device check of the token ids against the
 // vocabulary size V (V = 0: ids are trusted, as the reference trusts them).
 int encoder_launch(float* out, const int* inp, const float* wte, const float* wpe, int B, int T,

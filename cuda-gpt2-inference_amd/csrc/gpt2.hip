@@ -61,6 +61,15 @@ struct GPT2 {
   int kv_batch;  // sequences the cache is allocated for
   int kv_len;    // positions filled so far (the same for every sequence); 0 = empty
 
+  // the persistent decode-step kernel: barrier flags + error word on the device, the epoch
+  // its last launch ended with, a pinned host copy of the error word (refreshed after every
+  // step, looked at on the next call)
+  unsigned* step_flags;
+  unsigned step_epoch;
+  unsigned* step_error_host;
+  bool step_persistent;      // use the persistent kernel where it takes the model
+  unsigned step_spin_limit;  // polls of a barrier flag before a workgroup gives up
+
   // forward passes captured as HIP graphs, one per (B, T); they hold the activation
   // pointers, so they are dropped whenever the activations are reallocated
   struct Captured {
@@ -97,7 +106,11 @@ static void free_activations(GPT2* m) {
 static void free_cache(GPT2* m) {
   if (m->kv) (void)hipFree(m->kv);
   if (m->step_logits) (void)hipFree(m->step_logits);
+  if (m->step_flags) (void)hipFree(m->step_flags);
+  if (m->step_error_host) (void)hipHostFree(m->step_error_host);
   m->kv = m->step_logits = nullptr;
+  m->step_flags = m->step_error_host = nullptr;
+  m->step_epoch = 0;
   m->kv_batch = m->kv_len = 0;
 }
 
@@ -109,6 +122,11 @@ static int reserve_cache(GPT2* m, int B) {
   const size_t kv_bytes = (size_t)c.num_layers * 2 * B * c.max_seq_len * c.channels * sizeof(float);
   hipError_t e = hipMalloc((void**)&m->kv, kv_bytes);
   if (e == hipSuccess) e = hipMalloc((void**)&m->step_logits, (size_t)B * c.vocab_size * sizeof(float));
+  const size_t flag_bytes = decode_step_flag_bytes(m->device);
+  if (e == hipSuccess && flag_bytes) e = hipMalloc((void**)&m->step_flags, flag_bytes);
+  if (e == hipSuccess && flag_bytes) e = hipMemset(m->step_flags, 0, flag_bytes);
+  if (e == hipSuccess) e = hipHostMalloc((void**)&m->step_error_host, sizeof(unsigned), hipHostMallocDefault);
+  if (e == hipSuccess) *m->step_error_host = 0;
   if (e != hipSuccess) {
     free_cache(m);
     return fail(GPT2HIP_ENOMEM, "gpt2: key/value cache for %d sequences (%zu bytes): %s", B, kv_bytes,
@@ -261,6 +279,8 @@ GPT2* gpt2_create(const GPT2Config* config) {
   }
   GPT2* m = new GPT2();
   m->cfg = *config;
+  m->step_persistent = true;
+  m->step_spin_limit = 1u << 21;
   const size_t V = config->vocab_size, maxT = config->max_seq_len, L = config->num_layers,
                C = config->channels;
   const size_t sizes[P_COUNT] = {V * C,         maxT * C, L * C,         L * C,
@@ -509,9 +529,63 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device) {
   float* other = m->res_b;
   G2_HIP(hipMemcpyAsync(m->ids, next_ids_device, (size_t)B * sizeof(int), hipMemcpyDeviceToDevice,
                         stream()));
-  G2_TRY(encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
+  const bool persistent = m->step_persistent && m->step_flags && decode_step_supported(c, B, m->device);
+  if (!persistent)  // the persistent kernel gathers the embeddings itself
+    G2_TRY(encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
   const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
-  if (skinny_supported(B, C, true, residual, m->params) && skinny_supported(B, 4 * C, false, m->fch, m->params)) {
+  if (m->step_error_host && *m->step_error_host != 0) {
+    // an earlier step's kernel gave up a barrier wait: its logits and the cache row it was to
+    // append are not valid.  Clear the error so that a new prompt can run.
+    *m->step_error_host = 0;
+    G2_HIP(hipMemsetAsync(m->step_flags, 0, decode_step_flag_bytes(m->device), stream()));
+    m->step_epoch = 0;
+    m->kv_len = 0;
+    return fail(GPT2HIP_EHIP, "gpt2_decode: a workgroup of an earlier step gave up waiting at a grid "
+                              "barrier; the cache is invalid, prefill again");
+  }
+  if (persistent) {
+    // one persistent kernel for the whole step
+    DecodeStep st;
+    st.wte = P(P_WTE);
+    st.wpe_row = P(P_WPE) + (size_t)pos * cs;
+    st.ln1w = P(P_LN1W);
+    st.ln1b = P(P_LN1B);
+    st.qkvw = P(P_QKVW);
+    st.qkvb = P(P_QKVB);
+    st.attprojw = P(P_ATTPROJW);
+    st.attprojb = P(P_ATTPROJB);
+    st.ln2w = P(P_LN2W);
+    st.ln2b = P(P_LN2B);
+    st.fcw = P(P_FCW);
+    st.fcb = P(P_FCB);
+    st.fcprojw = P(P_FCPROJW);
+    st.fcprojb = P(P_FCPROJB);
+    st.lnfw = P(P_LNFW);
+    st.lnfb = P(P_LNFB);
+    st.ids = m->ids;
+    st.kv = m->kv;
+    st.plane = plane;
+    st.x = residual;
+    st.qkv = m->qkv;
+    st.atty = m->atty;
+    st.h = m->fch;
+    st.logits = m->step_logits;
+    st.flags = m->step_flags;
+    st.epoch0 = m->step_epoch;
+    st.spin_limit = m->step_spin_limit;
+    st.B = B;
+    st.C = C;
+    st.L = L;
+    st.NH = NH;
+    st.V = V;
+    st.pos = pos;
+    st.maxT = c.max_seq_len;
+    G2_TRY(decode_step_launch(st, c, m->device));
+    m->step_epoch += 5u * (unsigned)L + 8u;
+    G2_HIP(hipMemcpyAsync(m->step_error_host, (const char*)m->step_flags + decode_step_flag_bytes(m->device) -
+                                                  16 * sizeof(unsigned),
+                          sizeof(unsigned), hipMemcpyDeviceToHost, stream()));
+  } else if (skinny_supported(B, C, true, residual, m->params) && skinny_supported(B, 4 * C, false, m->fch, m->params)) {
     // Up to 16 sequences: five launches per block.  The layernorms run inside the GEMMs
     // that consume them and the residual adds inside the GEMMs that produce the update:
     //   qkv = LN1(x) Wqkv ; attention ; x += atty Wproj ; h = gelu(LN2(x) Wfc) ; x += h Wfcproj
@@ -556,6 +630,13 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device) {
 #undef G2_TRY
   m->kv_len = pos + 1;
   m->last_has_logits = false;  // the (B,T,V) buffer and the activations no longer describe a full pass
+  return GPT2HIP_OK;
+}
+
+int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit) {
+  if (!model) return g2::fail(GPT2HIP_EINVAL, "gpt2_decode_options: null model");
+  model->step_persistent = persistent != 0;
+  model->step_spin_limit = spin_limit;
   return GPT2HIP_OK;
 }
 
