@@ -315,6 +315,28 @@ def decode_bench(model, cfg, B, T0, steps):
            "ms_per_step": ms, "tokens_per_s": B / ms * 1e3,
            "bytes_per_step": weight_bytes + cache_bytes, "GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
            "finite": bool(torch.isfinite(model.step_logits()).all())}
+    try:
+        # one more step with the persistent kernel's clock probe: per phase kind, the mean time
+        # a workgroup works and the mean time from its arrival to everybody's arrival
+        clk = model.decode_probe(nxt[0]).cpu().numpy().astype("float64") * 10.0  # ns
+        names = ("qkv", "attention", "attproj", "fc_gelu", "fcproj")
+        done, passed = clk[:, 0, :], clk[:, 1, :]
+        start = clk[0, 0, :].min()
+        work = {n: [] for n in names}
+        wait = {n: [] for n in names}
+        prev = None
+        for p in range(5 * L):
+            begin = passed[p - 1] if p else None
+            if begin is not None:
+                work[names[p % 5]].append(float((done[p] - begin).mean()))
+            wait[names[p % 5]].append(float((passed[p] - done[p]).mean()))
+        row["probe_us"] = {
+            "kernel": float((done[5 * L].max() - start) / 1e3),
+            "lm_head": float((done[5 * L] - passed[5 * L - 1]).mean() / 1e3),
+            "work": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in work.items()},
+            "barrier": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in wait.items()}}
+    except g2.GPT2HipError:
+        pass
     log("  decode", json.dumps(row))
     return row
 

@@ -47,7 +47,8 @@ EXPORTS = (
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
     "gpt2_forward_device_status", "gpt2_forward_graph_status",
-    "gpt2_prefill_status", "gpt2_decode_status", "gpt2_decode_options", "gpt2_step_logits", "gpt2_cache_length",
+    "gpt2_prefill_status", "gpt2_decode_status", "gpt2_decode_options", "gpt2_decode_probe_status", "gpt2_decode_probe_size",
+    "gpt2_step_logits", "gpt2_cache_length",
     "gpt2_forward_argmax_status",
     "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
@@ -132,6 +133,8 @@ def lib() -> ctypes.CDLL:
         L.gpt2_prefill_status.argtypes, L.gpt2_prefill_status.restype = [vp, vp, ci, ci], ci
         L.gpt2_decode_status.argtypes, L.gpt2_decode_status.restype = [vp, vp], ci
         L.gpt2_decode_options.argtypes, L.gpt2_decode_options.restype = [vp, ci, ctypes.c_uint], ci
+        L.gpt2_decode_probe_status.argtypes, L.gpt2_decode_probe_status.restype = [vp, vp, vp, cz], ci
+        L.gpt2_decode_probe_size.argtypes, L.gpt2_decode_probe_size.restype = [vp], cz
         L.gpt2_step_logits.argtypes, L.gpt2_step_logits.restype = [vp], vp
         L.gpt2_cache_length.argtypes, L.gpt2_cache_length.restype = [vp], ci
         L.gpt2_forward_graph_status.argtypes = [vp, vp, ci, ci]
@@ -367,6 +370,20 @@ class GPT2:
             raise GPT2HipError("decode: expected one token id per prefilled sequence")
         _check(lib().gpt2_decode_status(self._h, _i32(next_ids_device)), "gpt2_decode")
         return self.step_logits()
+
+    def decode_probe(self, next_ids_device):
+        """One decode step of the persistent kernel with its clock probe: returns a
+        (phases, 2, workgroups) int64 tensor of 100 MHz wall-clock readings (work done / barrier
+        passed) -- see gpt2_decode_probe_status in the header."""
+        import torch
+        n = lib().gpt2_decode_probe_size(self._h)
+        if n == 0:
+            raise GPT2HipError("decode_probe: the persistent kernel does not take this model")
+        clocks = torch.zeros(n, dtype=torch.int64, device="cuda")
+        _check(lib().gpt2_decode_probe_status(self._h, _i32(next_ids_device), clocks.data_ptr(), n),
+               "gpt2_decode_probe")
+        phases = 5 * self.config.num_layers + 1
+        return clocks.view(phases, 2, -1)
 
     def decode_options(self, persistent: bool = True, spin_limit: int = 1 << 21):
         """Choose between the persistent decode-step kernel and one launch per operation."""

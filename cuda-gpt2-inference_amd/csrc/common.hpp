@@ -145,6 +145,9 @@ struct DecodeStep {
   unsigned* flags;            // [gridDim.x * FLAG_STRIDE] epochs, then the error word
   unsigned epoch0;            // flags hold values below epoch0 + 1 when the kernel starts
   unsigned spin_limit;
+  // optional probe: 100 MHz wall clock of every workgroup when it has finished phase p's work
+  // (trace[(2p) * G + g]) and when it has passed the barrier after it (trace[(2p+1) * G + g])
+  unsigned long long* trace;
   int B, C, L, NH, V, pos, maxT;
 };
 // Whether the persistent kernel takes the model at B sequences on this device; the bytes of

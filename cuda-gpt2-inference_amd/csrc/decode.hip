@@ -8,9 +8,9 @@
 // workgroups (~1.5 us, see below), and the next operation's weights are already on their
 // way into the L2 while the barrier is waited for.
 //
-// Work split.  Every workgroup (one per compute unit, 16 waves) takes N / gridDim.x
+// Work split.  Every workgroup (one per compute unit, 4 waves: one per SIMD) takes N / gridDim.x
 // consecutive weight rows (= output columns) of each GEMM for the whole K, at most 16 of
-// them: one 16x16 MFMA tile per workgroup whose K range is split over the 16 waves
+// them: one 16x16 MFMA tile per workgroup whose K range is split over the 4 waves
 // (v_mfma_f32_16x16x4_f32, A = 16 weight rows, B = the <= 16 activation rows; partial
 // tiles summed through LDS in wave order, so results are deterministic).  No output is
 // shared between workgroups and nothing is reduced through memory.  The layernorms run
@@ -20,6 +20,9 @@
 // epilogue:
 //   qkv = LN1(x) Wqkv | attention over the cache | x += y Wproj | h = gelu(LN2(x) Wfc) |
 //   x += h Wfcproj
+// (Four waves, not sixteen: a phase is a few hundred instructions of bookkeeping per wave
+// around a few dozen loads and MFMAs, every wave repeats the bookkeeping, and with sixteen
+// waves that repetition -- not memory -- set the pace: 5.4 us per layernorm+GEMM phase.)
 // Attention takes one workgroup per (sequence, head): it appends the new key and value to
 // the cache and runs the softmax over positions 0..pos, 16 lanes per cache row.
 // The lm-head gives every wave 16-row groups of wte for the whole K (no cross-wave sum),
@@ -40,15 +43,15 @@
 
 namespace g2 {
 
-constexpr int DS_WAVES = 16;
+constexpr int DS_WAVES = 4;
 constexpr int DS_THREADS = DS_WAVES * kWave;
-constexpr int DS_PF = 12;      // K units (16 floats x 16 rows) of weights a wave holds in registers
+constexpr int TRACE_SLOTS = 8;
 constexpr int FLAG_STRIDE = 16;  // one 64-byte line per workgroup's flag
 
 // LDS carve-up, in floats
-constexpr int LDS_RED = 0;                                // [16 waves][4][64] partial tiles
-constexpr int LDS_STAT = LDS_RED + DS_WAVES * 4 * kWave;  // [2][16 waves][16 rows]
-constexpr int LDS_SMALL = LDS_STAT + 2 * DS_WAVES * 16;   // [2][16]: attention max / sum per wave
+constexpr int LDS_RED = 0;                                // [waves][4][64] partial tiles
+constexpr int LDS_STAT = LDS_RED + DS_WAVES * 4 * kWave;  // [2][waves][16 rows]
+constexpr int LDS_SMALL = LDS_STAT + 2 * DS_WAVES * 16;   // [2][waves]: attention max / sum per wave
 constexpr int LDS_BAD = LDS_SMALL + 2 * DS_WAVES;         // one int: a wait timed out
 constexpr int LDS_SINK = LDS_BAD + 32;                    // 1 KiB that prefetches write and nobody reads
 constexpr int LDS_FREE = LDS_SINK + 256;                  // attention scores | lm-head activations
@@ -59,6 +62,10 @@ __device__ __forceinline__ f32x4 load_bypass4(const float* p) {
   f32x4 v;
   asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
   return v;  // not valid before wait_vm() + pin()
+}
+// The same into a register that already holds a value: lanes that are switched off keep it.
+__device__ __forceinline__ void load_bypass4_into(f32x4& v, const float* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "+v"(v) : "v"(p) : "memory");
 }
 __device__ __forceinline__ void store_bypass4(float* p, f32x4 v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
@@ -88,7 +95,12 @@ __device__ __forceinline__ int opaque_tid() {
 
 // ---- grid barrier ---------------------------------------------------------------------------
 // arrive(): this workgroup's stores of the phase are acknowledged, its flag shows `epoch`.
+__device__ __forceinline__ void trace_mark(const DecodeStep& a, unsigned phase, int k) {
+  if (a.trace != nullptr && threadIdx.x == 0)
+    a.trace[(size_t)(TRACE_SLOTS * phase + k) * gridDim.x + blockIdx.x] = wall_clock64();
+}
 __device__ __forceinline__ void grid_arrive(const DecodeStep& a, unsigned epoch) {
+  trace_mark(a, epoch - a.epoch0 - 1, 0);
   wait_vm();
   __syncthreads();
   if (threadIdx.x == 0)
@@ -115,17 +127,10 @@ __device__ __forceinline__ bool grid_wait(const DecodeStep& a, float* lds, unsig
     }
   }
   lds_barrier();
+  trace_mark(a, epoch - a.epoch0 - 1, 1);
   return *bad == 0;
 }
 
-// A wave's share of K, in units of 16 floats.
-struct Slice {
-  int u0, cnt;
-};
-__device__ __forceinline__ Slice wave_slice(int K, int wave) {
-  const int units = K >> 4, per = units / DS_WAVES, rem = units % DS_WAVES;
-  return {wave * per + min(wave, rem), per + (wave < rem ? 1 : 0)};
-}
 // A workgroup's share of the N output columns.
 struct Rows {
   int n0, nrows;
@@ -136,145 +141,183 @@ __device__ __forceinline__ Rows wg_rows(int N) {
   return {n0, min(rp, N - n0)};
 }
 
-// Warms the L2 of this workgroup's XCD with the weights the workgroup will read in its next
-// GEMM phase: the same addresses as weight_ptr() below, fetched by loads that write to a
-// scrap KiB of LDS (global_load_lds_dwordx4: no destination registers that a late-landing
-// load could clobber).  Issued right after the workgroup has arrived at a grid barrier, so
-// that HBM latency runs while the barrier is waited for; the phase's own loads then hit the L2.
+// Warming the L2 of this workgroup's XCD with what the workgroup reads in its next phase:
+// loads that write to a scrap KiB of LDS (global_load_lds_dwordx4: no destination registers
+// that a late-landing load could clobber).  Issued right after the workgroup has arrived at
+// a grid barrier, so that HBM latency runs while the barrier is waited for; the phase's own
+// loads then hit the L2.
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
 __device__ __forceinline__ void touch(const float* p, float* lds) {
   __builtin_amdgcn_global_load_lds((glb_void_t*)p, (lds_void_t*)(lds + LDS_SINK), 16, 0, 0);
 }
-__device__ __forceinline__ const float* weight_ptr(const float* W, const Rows& r, const Slice& s, int K,
-                                                   int lane) {
-  // rows past the workgroup's share repeat its last row: they feed result columns that are not stored
-  return W + (size_t)(r.n0 + min(lane & 15, r.nrows - 1)) * K + (size_t)s.u0 * 16 + 4 * (lane >> 4);
+// n floats from p, 1 KiB per wave instruction, spread over the waves.
+__device__ __forceinline__ void prefetch_span(float* lds, const float* p, int n, int pw, int lane) {
+  for (int i = pw * 256 + lane * 4; i < n; i += DS_WAVES * 256) touch(p + i, lds);
 }
-// U: units of K per wave.
-template <int U>
-__device__ __forceinline__ void prefetch_weights(float* lds, const float* W, int N, int K) {
-  const int tid = opaque_tid();
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+// The weight rows, bias and layernorm parameters of a GEMM phase.
+__device__ __forceinline__ void prefetch_gemm(float* lds, const float* W, const float* bias, int N, int K,
+                                              const float* ln_w, const float* ln_b) {
+  const int tid = opaque_tid(), lane = tid & 63;
+  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6);
   const Rows r = wg_rows(N);
   if (r.nrows <= 0) return;
-  const Slice s = wave_slice(K, wave);
-  const float* wp = weight_ptr(W, r, s, K, tid & 63);
-#pragma unroll
-  for (int c = 0; c < U; c++) touch(wp + c * 16, lds);
+  const float* wp = W + (size_t)(r.n0 + min(lane & 15, r.nrows - 1)) * K + 4 * (lane >> 4);
+  const int units = K >> 4;
+  for (int u = pw; u < units; u += DS_WAVES) touch(wp + (size_t)u * 16, lds);
+  if (ln_w != nullptr) {
+    prefetch_span(lds, ln_w, K, pw, lane);
+    prefetch_span(lds, ln_b, K, pw, lane);
+  }
+  if (bias != nullptr && pw == 0 && lane < 5) {
+    // the 16-byte pieces that hold bias[n0 .. n0 + nrows): at most five
+    const float* b0 = bias + ((r.n0 & ~3) + 4 * lane);
+    if (b0 < bias + r.n0 + r.nrows) touch(b0, lds);
+  }
+}
+// The cache rows attention_item() will read for this workgroup's first (sequence, head): up to
+// 24 wave instructions (4 rows of 256 bytes each) of keys and as many of values per wave.
+__device__ __forceinline__ void prefetch_cache(const DecodeStep& a, float* lds, const float* kc,
+                                               const float* vc) {
+  const int tid = opaque_tid(), lane = tid & 63;
+  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int item = blockIdx.x;
+  if (item >= a.B * a.NH || a.pos < 1) return;
+  const int b = item / a.NH, head = item % a.NH;
+  const size_t off = (size_t)b * a.maxT * a.C + head * 64 + 4 * (lane & 15);
+  const int last = a.pos - 1;  // rows 0..pos-1 exist; row pos is written by the phase itself
+  for (int i = 0; i < 24; i++) {
+    const int t0 = 4 * (pw + DS_WAVES * i);
+    if (t0 > last) break;
+    const size_t row = (size_t)min(t0 + (lane >> 4), last) * a.C;
+    touch(kc + off + row, lds);
+    touch(vc + off + row, lds);
+  }
 }
 
 // out[j][n0 + i] = resid + act( LN(in)[j] . W[n0 + i] + bias ) for this workgroup's columns.
+// A wave's share of K is NCH chunks of U units; a chunk's loads are all issued at once.
+// (NCH > 1 only without LN, whose statistics need the wave's whole share in registers.)
 // GATHER: the input rows are wte[ids[j]] + wpe[pos] (the first phase of a step); workgroup 0
 // also stores them as the residual stream x.
-template <bool LN, bool GELU, bool GATHER, int U>
+template <bool LN, bool GELU, bool GATHER, int U, int NCH>
 __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, const float* __restrict__ W,
                                            const float* __restrict__ bias, int N, int K,
                                            const float* in, const float* __restrict__ ln_w,
                                            const float* __restrict__ ln_b, float* out,
-                                           const float* resid) {
+                                           const float* resid, unsigned ph = 0) {
+  static_assert(!LN || NCH == 1, "a normalised row is held whole");
   const int tid = opaque_tid(), lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kq = lane >> 4;
   const Rows r = wg_rows(N);
   if (r.nrows <= 0) return;  // the whole workgroup
-  const Slice s = wave_slice(K, wave);
   const int B = a.B;
   // epilogue element of this thread: column n0 + oi of row oj
   const int oi = tid & 15, oj = tid >> 4;
-  const bool owner = tid < 256 && oi < r.nrows && oj < B;
+  const bool owner = oi < r.nrows && oj < B;
   float rs = 0.f, bs = 0.f;
   if (owner) {
     if (resid != nullptr) rs = load_bypass(resid + (size_t)oj * N + r.n0 + oi);
     if (bias != nullptr) bs = bias[r.n0 + oi];
   }
 
-  constexpr int NX = U;
-  const int jr = min(r16, B - 1);
-  const size_t koff = (size_t)s.u0 * 16 + 4 * kq;
-  f32x4 wv[NX], xv[NX], gv[LN ? NX : 1], bv[LN ? NX : 1];
-  {
-    const float* wp = weight_ptr(W, r, s, K, lane);
-#pragma unroll
-    for (int c = 0; c < NX; c++)
-      wv[c] = *reinterpret_cast<const f32x4*>(wp + c * 16);
-  }
-  if (GATHER) {
-    const int id = a.ids[jr];
-    const bool ok = (unsigned)id < (unsigned)a.V;
-    const float* tp = a.wte + (size_t)(ok ? id : 0) * K + koff;
-    const float* pp = a.wpe_row + koff;
-    const float q = __builtin_nanf("");
-#pragma unroll
-    for (int c = 0; c < NX; c++)
-      {
-        xv[c] = *reinterpret_cast<const f32x4*>(tp + c * 16) + *reinterpret_cast<const f32x4*>(pp + c * 16);
-        if (!ok) xv[c] = f32x4{q, q, q, q};
-        if (blockIdx.x == 0 && r16 < B) store_bypass4(a.x + (size_t)r16 * K + koff + c * 16, xv[c]);
-      }
-  } else {
-    const float* xp = in + (size_t)jr * K + koff;
-#pragma unroll
-    for (int c = 0; c < NX; c++)
-      xv[c] = load_bypass4(xp + c * 16);
-  }
+  // this lane's first float of the wave's share of K
+  const size_t koff = (size_t)wave * (U * NCH * 16) + 4 * kq;
+  const float* wp = W + (size_t)(r.n0 + r16) * K + koff;
+  // Loads cost the compute unit's one load path 64 bytes per cycle whether or not lanes
+  // repeat each other's addresses, so lanes beyond the workgroup's weight rows / beyond the
+  // B activation rows are switched off (their operands are zero) instead of clamped, and
+  // the layernorm's gamma and beta, which every row shares, go through LDS.
+  float* const gb = lds + LDS_FREE;  // gamma [K] | beta [K]
   if (LN) {
+    for (int i = tid * 4; i < K; i += DS_THREADS * 4) {
+      *reinterpret_cast<f32x4*>(gb + i) = *reinterpret_cast<const f32x4*>(ln_w + i);
+      *reinterpret_cast<f32x4*>(gb + K + i) = *reinterpret_cast<const f32x4*>(ln_b + i);
+    }
+  }
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < NX; c++)
-      {
-        gv[c] = *reinterpret_cast<const f32x4*>(ln_w + koff + c * 16);
-        bv[c] = *reinterpret_cast<const f32x4*>(ln_b + koff + c * 16);
+  for (int ch = 0; ch < NCH; ch++) {
+    f32x4 wv[U], xv[U];
+#pragma unroll
+    for (int c = 0; c < U; c++) {
+      wv[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+      xv[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (r16 < r.nrows) {
+#pragma unroll
+      for (int c = 0; c < U; c++) wv[c] = *reinterpret_cast<const f32x4*>(wp + (ch * U + c) * 16);
+    }
+    if (GATHER) {
+      if (r16 < B) {
+        const int id = a.ids[r16];
+        const bool ok = (unsigned)id < (unsigned)a.V;
+        const float* tp = a.wte + (size_t)(ok ? id : 0) * K + koff;
+        const float* pp = a.wpe_row + koff;
+        const float q = __builtin_nanf("");
+#pragma unroll
+        for (int c = 0; c < U; c++) {
+          xv[c] = *reinterpret_cast<const f32x4*>(tp + c * 16) + *reinterpret_cast<const f32x4*>(pp + c * 16);
+          if (!ok) xv[c] = f32x4{q, q, q, q};
+          if (blockIdx.x == 0) store_bypass4(a.x + (size_t)r16 * K + koff + c * 16, xv[c]);
+        }
       }
-  }
-  if (!GATHER) {
-    wait_vm();
+    } else {
+      if (r16 < B) {
+        const float* xp = in + (size_t)r16 * K + koff;
 #pragma unroll
-    for (int c = 0; c < NX; c++)
-      pin(xv[c]);
-  }
+        for (int c = 0; c < U; c++) load_bypass4_into(xv[c], xp + (ch * U + c) * 16);
+      }
+      if (ch == 0) trace_mark(a, ph, 2);
+      wait_vm();
+#pragma unroll
+      for (int c = 0; c < U; c++) pin(xv[c]);
+      if (ch == 0) trace_mark(a, ph, 3);
+    }
 
-  if (LN) {
-    // row r16's statistics: lanes r16 + 16*kq of all 16 waves hold the row between them
-    float* const stat = lds + LDS_STAT;
-    float sum = 0.f;
+    if (LN) {
+      // row r16's statistics: lanes r16 + 16*kq of all the waves hold the row between them
+      float* const stat = lds + LDS_STAT;
+      float sum = 0.f;
 #pragma unroll
-    for (int c = 0; c < NX; c++)
-      sum += (xv[c][0] + xv[c][1]) + (xv[c][2] + xv[c][3]);
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
-    if (kq == 0) stat[wave * 16 + r16] = sum;
-    __syncthreads();
-    float mean = 0.f;
+      for (int c = 0; c < U; c++) sum += (xv[c][0] + xv[c][1]) + (xv[c][2] + xv[c][3]);
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      if (kq == 0) stat[wave * 16 + r16] = sum;
+      __syncthreads();
+      float mean = 0.f;
 #pragma unroll
-    for (int w = 0; w < DS_WAVES; w++) mean += stat[w * 16 + r16];
-    mean /= (float)K;
-    float q = 0.f;
+      for (int w = 0; w < DS_WAVES; w++) mean += stat[w * 16 + r16];
+      mean /= (float)K;
+      float q = 0.f;
 #pragma unroll
-    for (int c = 0; c < NX; c++)
-      {
+      for (int c = 0; c < U; c++) {
         const f32x4 d = xv[c] - mean;
         q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
       }
-    q += __shfl_xor(q, 16, 64);
-    q += __shfl_xor(q, 32, 64);
-    if (kq == 0) stat[DS_WAVES * 16 + wave * 16 + r16] = q;
-    __syncthreads();
-    float var = 0.f;
+      q += __shfl_xor(q, 16, 64);
+      q += __shfl_xor(q, 32, 64);
+      if (kq == 0) stat[DS_WAVES * 16 + wave * 16 + r16] = q;
+      __syncthreads();
+      float var = 0.f;
 #pragma unroll
-    for (int w = 0; w < DS_WAVES; w++) var += stat[DS_WAVES * 16 + w * 16 + r16];
-    const float rstd = 1.0f / sqrtf(var / (float)K + 1e-5f);
+      for (int w = 0; w < DS_WAVES; w++) var += stat[DS_WAVES * 16 + w * 16 + r16];
+      const float rstd = 1.0f / sqrtf(var / (float)K + 1e-5f);
 #pragma unroll
-    for (int c = 0; c < NX; c++)
-      xv[c] = (xv[c] - mean) * rstd * gv[c] + bv[c];
-  }
+      for (int c = 0; c < U; c++)
+        xv[c] = (xv[c] - mean) * rstd * *reinterpret_cast<const f32x4*>(gb + koff + c * 16) +
+                *reinterpret_cast<const f32x4*>(gb + K + koff + c * 16);
+      trace_mark(a, ph, 4);
+    }
 
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int c = 0; c < NX; c++)
-    {
+    for (int c = 0; c < U; c++) {
 #pragma unroll
       for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[c][e], xv[c][e], acc, 0, 0, 0);
     }
+  }
+  trace_mark(a, ph, 5);
   // lane l holds D[4*(l/16) + v][l % 16]: weight row (output column) 4*(l/16)+v, activation row l%16
   float* const red = lds + LDS_RED;
 #pragma unroll
@@ -294,11 +337,11 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
 
 // One (sequence, head) of attention against the cache, head size 64: appends the new key and
 // value (taken from the qkv row other workgroups just wrote), scores positions 0..pos with
-// 16 lanes per cache row (a wave instruction covers four positions, 8 of them in flight),
+// 16 lanes per cache row (a wave instruction covers four positions, 16 of them in flight),
 // softmax through LDS, weighted values the same way.
 __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, float* kc, float* vc,
                                                int b, int head) {
-  constexpr int UN = 8;
+  constexpr int UN = 16;
   const int tid = opaque_tid(), lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int p4 = lane >> 4, sub = lane & 15;
@@ -395,26 +438,27 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
 }
 
 // logits = LNf(x) . wte^T.  The normalised rows go to LDS once per workgroup; wave w then
-// takes the 16-row groups g + gridDim.x * (w + 16 i) of wte for the whole K; the first units of
-// its first group were requested into the L2 before the last barrier.
-__device__ __forceinline__ void lm_head_first_group(int& cg, int wave) {
-  cg = (int)blockIdx.x + (int)gridDim.x * wave;
+// takes the 16-row groups g + gridDim.x * (w + 4 i) of wte for the whole K, UC units at a
+// time; the first units of its first group were requested into the L2 before the last barrier.
+__device__ __forceinline__ int lm_head_first_group(int wave) {
+  return (int)blockIdx.x + (int)gridDim.x * wave;
 }
-template <int U>
+template <int UC>
 __device__ __forceinline__ void prefetch_lm_head(const DecodeStep& a, float* lds) {
   const int tid = opaque_tid(), lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  int cg;
-  lm_head_first_group(cg, wave);
-  if (cg * 16 >= a.V) return;
   const int K = a.C;
+  prefetch_span(lds, a.lnfw, K, wave, lane);
+  prefetch_span(lds, a.lnfb, K, wave, lane);
+  const int cg = lm_head_first_group(wave);
+  if (cg * 16 >= a.V) return;
   const float* wp = a.wte + (size_t)min(cg * 16 + (lane & 15), a.V - 1) * K + 4 * (lane >> 4);
-  const int units = K >> 4;
 #pragma unroll
-  for (int c = 0; c < U; c++) touch(wp + c * 16, lds);
+  for (int c = 0; c < UC; c++) touch(wp + c * 16, lds);
 }
 
-// U1: units of K per wave in the layernorm; UC: units per chunk of a wave's sweep over K.
+// U1: units of K per wave in the layernorm (K = 64 * U1); UC: units per chunk of a wave's sweep
+// over K (a divisor of 4 * U1).
 template <int U1, int UC>
 __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   const int tid = opaque_tid(), lane = tid & 63;
@@ -424,29 +468,27 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   const int ldx = K + 4;  // row stride of the staged activations
   float* const xs = lds + LDS_FREE;
   {
-    const Slice s = wave_slice(K, wave);
-    const int jr = min(r16, B - 1);
-    const size_t koff = (size_t)s.u0 * 16 + 4 * kq;
-    const float* xp = a.x + (size_t)jr * K + koff;
-    f32x4 xv[U1], gv[U1], bv[U1];
+    const size_t koff = (size_t)wave * (U1 * 16) + 4 * kq;
+    float* const gb = xs + (size_t)B * ldx;  // gamma [K] | beta [K], shared by all rows
+    for (int i = tid * 4; i < K; i += DS_THREADS * 4) {
+      *reinterpret_cast<f32x4*>(gb + i) = *reinterpret_cast<const f32x4*>(a.lnfw + i);
+      *reinterpret_cast<f32x4*>(gb + K + i) = *reinterpret_cast<const f32x4*>(a.lnfb + i);
+    }
+    f32x4 xv[U1];
 #pragma unroll
-    for (int c = 0; c < U1; c++)
-      xv[c] = load_bypass4(xp + c * 16);
+    for (int c = 0; c < U1; c++) xv[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (r16 < B) {
+      const float* xp = a.x + (size_t)r16 * K + koff;
 #pragma unroll
-    for (int c = 0; c < U1; c++)
-      {
-        gv[c] = *reinterpret_cast<const f32x4*>(a.lnfw + koff + c * 16);
-        bv[c] = *reinterpret_cast<const f32x4*>(a.lnfb + koff + c * 16);
-      }
+      for (int c = 0; c < U1; c++) load_bypass4_into(xv[c], xp + c * 16);
+    }
     wait_vm();
 #pragma unroll
-    for (int c = 0; c < U1; c++)
-      pin(xv[c]);
+    for (int c = 0; c < U1; c++) pin(xv[c]);
     float* const stat = lds + LDS_STAT;
     float sum = 0.f;
 #pragma unroll
-    for (int c = 0; c < U1; c++)
-      sum += (xv[c][0] + xv[c][1]) + (xv[c][2] + xv[c][3]);
+    for (int c = 0; c < U1; c++) sum += (xv[c][0] + xv[c][1]) + (xv[c][2] + xv[c][3]);
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     if (kq == 0) stat[wave * 16 + r16] = sum;
@@ -457,11 +499,10 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
     mean /= (float)K;
     float q = 0.f;
 #pragma unroll
-    for (int c = 0; c < U1; c++)
-      {
-        const f32x4 d = xv[c] - mean;
-        q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
-      }
+    for (int c = 0; c < U1; c++) {
+      const f32x4 d = xv[c] - mean;
+      q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+    }
     q += __shfl_xor(q, 16, 64);
     q += __shfl_xor(q, 32, 64);
     if (kq == 0) stat[DS_WAVES * 16 + wave * 16 + r16] = q;
@@ -470,35 +511,35 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
 #pragma unroll
     for (int w = 0; w < DS_WAVES; w++) var += stat[DS_WAVES * 16 + w * 16 + r16];
     const float rstd = 1.0f / sqrtf(var / (float)K + 1e-5f);
+    if (r16 < B) {
 #pragma unroll
-    for (int c = 0; c < U1; c++)
-      if (r16 < B)
+      for (int c = 0; c < U1; c++)
         *reinterpret_cast<f32x4*>(xs + (size_t)r16 * ldx + koff + c * 16) =
-            (xv[c] - mean) * rstd * gv[c] + bv[c];
+            (xv[c] - mean) * rstd * *reinterpret_cast<const f32x4*>(gb + koff + c * 16) +
+            *reinterpret_cast<const f32x4*>(gb + K + koff + c * 16);
+    }
     __syncthreads();
   }
 
-  const int units = K >> 4;
+  constexpr int NCH = 4 * U1 / UC;
+  static_assert(NCH * UC == 4 * U1, "UC must divide the units of K");
   const float* const xrow = xs + (size_t)min(r16, B - 1) * ldx + 4 * kq;
-  int cg;
-  lm_head_first_group(cg, wave);
-  for (; cg * 16 < V; cg += (int)gridDim.x * DS_WAVES) {
+  for (int cg = lm_head_first_group(wave); cg * 16 < V; cg += (int)gridDim.x * DS_WAVES) {
     const int n0 = cg * 16;
     const float* wp = a.wte + (size_t)min(n0 + r16, V - 1) * K + 4 * kq;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int u = 0; u < units; u += UC) {
+#pragma unroll 1
+    for (int ch = 0; ch < NCH; ch++) {
       f32x4 wv[UC];
 #pragma unroll
       for (int c = 0; c < UC; c++)
-        
-          wv[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)(u + c) * 16));
+        wv[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)(ch * UC + c) * 16));
 #pragma unroll
-      for (int c = 0; c < UC; c++)
-        {
-          const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + (u + c) * 16);
+      for (int c = 0; c < UC; c++) {
+        const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + (ch * UC + c) * 16);
 #pragma unroll
-          for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[c][e], xq[e], acc, 0, 0, 0);
-        }
+        for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[c][e], xq[e], acc, 0, 0, 0);
+      }
     }
     if (r16 < B) {
       float* op = a.logits + (size_t)r16 * V + n0 + 4 * kq;
@@ -509,9 +550,10 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   }
 }
 
-// U1 / U4: units of K (16 floats) per wave where K = C / K = 4C; C is a multiple of 256, so
-// every wave has exactly that many and the loops carry no guards.
-template <int U1, int U4>
+// U1: units of K (16 floats) per wave where K = C (C = 64 * U1, so every wave has exactly that
+// many and the loops carry no guards); where K = 4C a wave takes N4 chunks of U4 units
+// (U4 * N4 = 4 * U1).  ULM: units per chunk of the lm-head's sweep.
+template <int U1, int U4, int N4, int ULM>
 __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeStep a) {
   extern __shared__ float lds[];
   const int C = a.C;
@@ -529,13 +571,13 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
   for (int l = 0; l < a.L; l++) {
     // qkv = LN1(x) Wqkv + b
     if (l == 0)
-      gemm_phase<true, false, true, U1>(a, lds, a.qkvw, a.qkvb, 3 * C, C, nullptr, a.ln1w, a.ln1b,
-                                               a.qkv, nullptr);
+      gemm_phase<true, false, true, U1, 1>(a, lds, a.qkvw, a.qkvb, 3 * C, C, nullptr, a.ln1w, a.ln1b,
+                                               a.qkv, nullptr, epoch - a.epoch0);
     else
-      gemm_phase<true, false, false, U1>(a, lds, a.qkvw + l * 3 * cs * cs, a.qkvb + l * 3 * cs, 3 * C,
-                                                C, a.x, a.ln1w + l * cs, a.ln1b + l * cs, a.qkv, nullptr);
+      gemm_phase<true, false, false, U1, 1>(a, lds, a.qkvw + l * 3 * cs * cs, a.qkvb + l * 3 * cs, 3 * C,
+                                                C, a.x, a.ln1w + l * cs, a.ln1b + l * cs, a.qkv, nullptr, epoch - a.epoch0);
     grid_arrive(a, ++epoch);
-    prefetch_weights<U1>(lds, a.attprojw + l * cs * cs, C, C);
+    prefetch_cache(a, lds, a.kv + (2 * (size_t)l) * a.plane, a.kv + (2 * (size_t)l + 1) * a.plane);
     if (!grid_wait(a, lds, epoch)) return;
 
     // attention over the cache
@@ -543,33 +585,36 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
       attention_item(a, lds, a.kv + (2 * (size_t)l) * a.plane, a.kv + (2 * (size_t)l + 1) * a.plane,
                      item / a.NH, item % a.NH);
     grid_arrive(a, ++epoch);
+    prefetch_gemm(lds, a.attprojw + l * cs * cs, a.attprojb + l * cs, C, C, nullptr, nullptr);
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += y Wproj + b
-    gemm_phase<false, false, false, U1>(a, lds, a.attprojw + l * cs * cs, a.attprojb + l * cs, C, C,
-                                               a.atty, nullptr, nullptr, a.x, a.x);
+    gemm_phase<false, false, false, U1, 1>(a, lds, a.attprojw + l * cs * cs, a.attprojb + l * cs, C, C,
+                                               a.atty, nullptr, nullptr, a.x, a.x, epoch - a.epoch0);
     grid_arrive(a, ++epoch);
-    prefetch_weights<U1>(lds, a.fcw + l * 4 * cs * cs, 4 * C, C);
+    prefetch_gemm(lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, 4 * C, C, a.ln2w + l * cs, a.ln2b + l * cs);
     if (!grid_wait(a, lds, epoch)) return;
 
     // h = gelu(LN2(x) Wfc + b)
-    gemm_phase<true, true, false, U1>(a, lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, 4 * C, C,
-                                             a.x, a.ln2w + l * cs, a.ln2b + l * cs, a.h, nullptr);
+    gemm_phase<true, true, false, U1, 1>(a, lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, 4 * C, C,
+                                             a.x, a.ln2w + l * cs, a.ln2b + l * cs, a.h, nullptr, epoch - a.epoch0);
     grid_arrive(a, ++epoch);
-    prefetch_weights<U4>(lds, a.fcprojw + l * 4 * cs * cs, C, 4 * C);
+    prefetch_gemm(lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, C, 4 * C, nullptr, nullptr);
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += h Wfcproj + b
-    gemm_phase<false, false, false, U4>(a, lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, C,
-                                               4 * C, a.h, nullptr, nullptr, a.x, a.x);
+    gemm_phase<false, false, false, U4, N4>(a, lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, C,
+                                               4 * C, a.h, nullptr, nullptr, a.x, a.x, epoch - a.epoch0);
     grid_arrive(a, ++epoch);
     if (l + 1 < a.L)
-      prefetch_weights<U1>(lds, a.qkvw + (l + 1) * 3 * cs * cs, 3 * C, C);
+      prefetch_gemm(lds, a.qkvw + (l + 1) * 3 * cs * cs, a.qkvb + (l + 1) * 3 * cs, 3 * C, C,
+                    a.ln1w + (l + 1) * cs, a.ln1b + (l + 1) * cs);
     else
-      prefetch_lm_head<U4>(a, lds);
+      prefetch_lm_head<ULM>(a, lds);
     if (!grid_wait(a, lds, epoch)) return;
   }
-  lm_head_phase<U1, U4>(a, lds);
+  lm_head_phase<U1, ULM>(a, lds);
+  trace_mark(a, 5u * (unsigned)a.L, 0);
 }
 
 // ---- host ---------------------------------------------------------------------------------
@@ -589,7 +634,7 @@ size_t decode_step_flag_bytes(int device) {
 
 static size_t decode_step_lds_bytes(const GPT2Config& c, int B, int pos) {
   const size_t att = (size_t)((pos + 64) & ~63) + DS_WAVES * 64;
-  const size_t lm = (size_t)B * (c.channels + 4);
+  const size_t lm = (size_t)B * (c.channels + 4) + 2 * (size_t)c.channels;  // rows | gamma | beta
   return (LDS_FREE + (att > lm ? att : lm)) * sizeof(float);
 }
 
@@ -597,8 +642,8 @@ bool decode_step_supported(const GPT2Config& c, int B, int device) {
   const int C = c.channels, G = decode_step_workgroups(device);
   if (G < 1 || G > DS_THREADS) return false;
   if (B < 1 || B > 16 || c.num_heads * 64 != C) return false;
-  // every wave takes exactly C/256 (4C/256) units of 16 floats of K, at most DS_PF of them
-  if (C % 256 != 0 || 4 * C / 256 > DS_PF) return false;
+  // every wave takes exactly C/64 (4C/64) units of 16 floats of K; instantiated sizes only
+  if (C != 64 && C != 128 && C != 256 && C != 512 && C != 768 && C != 1024) return false;
   if ((4 * C + G - 1) / G > 16) return false;  // the widest N: at most 16 weight rows per workgroup
   return decode_step_lds_bytes(c, B, c.max_seq_len - 1) <= 160 * 1024;
 }
@@ -606,16 +651,18 @@ bool decode_step_supported(const GPT2Config& c, int B, int device) {
 int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) {
   const int G = decode_step_workgroups(device);
   const size_t lds = decode_step_lds_bytes(c, step.B, step.pos);
-  // channels a multiple of 256: every wave has exactly C/256 (4C/256) units, guard-free loops
   const void* kernel;
   int slot;
-  switch (c.channels % 256 == 0 ? c.channels / 256 : 0) {
-    case 1: kernel = reinterpret_cast<const void*>(decode_step_kernel<1, 4>); slot = 1; break;
-    case 2: kernel = reinterpret_cast<const void*>(decode_step_kernel<2, 8>); slot = 2; break;
-    case 3: kernel = reinterpret_cast<const void*>(decode_step_kernel<3, 12>); slot = 3; break;
+  switch (c.channels) {
+    case 64: kernel = reinterpret_cast<const void*>(decode_step_kernel<1, 4, 1, 4>); slot = 0; break;
+    case 128: kernel = reinterpret_cast<const void*>(decode_step_kernel<2, 8, 1, 8>); slot = 1; break;
+    case 256: kernel = reinterpret_cast<const void*>(decode_step_kernel<4, 16, 1, 16>); slot = 2; break;
+    case 512: kernel = reinterpret_cast<const void*>(decode_step_kernel<8, 32, 1, 16>); slot = 3; break;
+    case 768: kernel = reinterpret_cast<const void*>(decode_step_kernel<12, 48, 1, 24>); slot = 4; break;
+    case 1024: kernel = reinterpret_cast<const void*>(decode_step_kernel<16, 32, 2, 32>); slot = 5; break;
     default: return fail(GPT2HIP_EINVAL, "decode step kernel: channels %d not supported", c.channels);
   }
-  static bool lds_raised[4] = {false, false, false, false};
+  static bool lds_raised[6] = {false, false, false, false, false, false};
   if (lds > 48 * 1024 && !lds_raised[slot]) {
     G2_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     lds_raised[slot] = true;

@@ -507,8 +507,38 @@ int gpt2_prefill_status(GPT2* model, const int* inputs_device, int B, int T) {
   return GPT2HIP_OK;
 }
 
+namespace g2 {
+static int decode_step(GPT2* model, const int* next_ids_device, unsigned long long* trace);
+}
+
 int gpt2_decode_status(GPT2* model, const int* next_ids_device) {
+  return g2::decode_step(model, next_ids_device, nullptr);
+}
+
+int gpt2_decode_probe_status(GPT2* model, const int* next_ids_device, unsigned long long* clocks_device,
+                             size_t capacity) {
   using namespace g2;
+  if (!model || !clocks_device) return fail(GPT2HIP_EINVAL, "gpt2_decode_probe: null pointer");
+  const size_t need = gpt2_decode_probe_size(model);
+  if (need == 0)
+    return fail(GPT2HIP_EINVAL, "gpt2_decode_probe: the persistent kernel does not take this model");
+  if (capacity < need)
+    return fail(GPT2HIP_EINVAL, "gpt2_decode_probe: %zu clock slots given, %zu needed", capacity, need);
+  return decode_step(model, next_ids_device, clocks_device);
+}
+
+size_t gpt2_decode_probe_size(const GPT2* model) {
+  using namespace g2;
+  if (!model || !model->step_persistent || model->kv_batch < 1 ||
+      !decode_step_supported(model->cfg, model->kv_batch, model->device))
+    return 0;
+  // the flag array holds one 64-byte line per workgroup and one for the error word
+  const size_t workgroups = decode_step_flag_bytes(model->device) / (16 * sizeof(unsigned)) - 1;
+  return workgroups * (8 * (5 * (size_t)model->cfg.num_layers + 1));
+}
+
+namespace g2 {
+static int decode_step(GPT2* model, const int* next_ids_device, unsigned long long* trace) {
   if (!model || !next_ids_device) return fail(GPT2HIP_EINVAL, "gpt2_decode: null pointer");
   GPT2* m = model;
   const GPT2Config& c = m->cfg;
@@ -573,6 +603,7 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device) {
     st.flags = m->step_flags;
     st.epoch0 = m->step_epoch;
     st.spin_limit = m->step_spin_limit;
+    st.trace = trace;
     st.B = B;
     st.C = C;
     st.L = L;
@@ -632,6 +663,7 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device) {
   m->last_has_logits = false;  // the (B,T,V) buffer and the activations no longer describe a full pass
   return GPT2HIP_OK;
 }
+}  // namespace g2
 
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit) {
   if (!model) return g2::fail(GPT2HIP_EINVAL, "gpt2_decode_options: null model");

@@ -207,6 +207,15 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device);
  * spends on one flag of its grid barrier before it gives up and ends the kernel (default
  * 2^21); a step that gave up makes the NEXT gpt2_decode call fail and empties the cache. */
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit);
+/* One gpt2_decode step of the persistent kernel with a clock probe: every workgroup g records
+ * the 100 MHz wall clock when it has finished the work of phase p (clocks[(2p) * G + g]) and
+ * when it has passed the grid barrier after it (clocks[(2p + 1) * G + g]); phases are, per
+ * layer, qkv GEMM, attention, projection GEMM, fc GEMM, fc projection GEMM, then the lm-head
+ * (work only).  G = compute units of the device; gpt2_decode_probe_size() = the slots needed
+ * (0 if the persistent kernel does not take the model at the prefilled batch size). */
+int gpt2_decode_probe_status(GPT2* model, const int* next_ids_device, unsigned long long* clocks_device,
+                             size_t capacity);
+size_t gpt2_decode_probe_size(const GPT2* model);
 const float* gpt2_step_logits(const GPT2* model);
 int gpt2_cache_length(const GPT2* model);
 
