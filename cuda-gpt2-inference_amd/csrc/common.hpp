@@ -145,8 +145,9 @@ struct DecodeStep {
   unsigned* flags;            // [gridDim.x * FLAG_STRIDE] epochs, then the error word
   unsigned epoch0;            // flags hold values below epoch0 + 1 when the kernel starts
   unsigned spin_limit;
-  // optional probe: 100 MHz wall clock of every workgroup when it has finished phase p's work
-  // (trace[(2p) * G + g]) and when it has passed the barrier after it (trace[(2p+1) * G + g])
+  // optional probe: 100 MHz wall clock of every workgroup g of the G = 256 when it has finished
+  // phase p's work (trace[(2p) * G + g]) and when it has passed the barrier after it
+  // (trace[(2p+1) * G + g])
   unsigned long long* trace;
   int B, C, L, NH, V, pos, maxT;
 };
@@ -155,6 +156,7 @@ struct DecodeStep {
 // uses barrier epochs step.epoch0 + 1 .. step.epoch0 + 5 * L.
 bool decode_step_supported(const GPT2Config& c, int B, int device);
 size_t decode_step_flag_bytes(int device);
+size_t decode_step_probe_slots(int num_layers);  // clock slots DecodeStep::trace needs
 int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device);
 
 // encoder_forward with an optional on-device check of the token ids against the

@@ -45,34 +45,39 @@ namespace g2 {
 
 constexpr int DS_WAVES = 4;
 constexpr int DS_THREADS = DS_WAVES * kWave;
-constexpr int TRACE_SLOTS = 8;
+constexpr int TRACE_SLOTS = 2;
+constexpr int DS_GRID = 256;  // workgroups: the shapes below are compiled for exactly this many
 constexpr int FLAG_STRIDE = 16;  // one 64-byte line per workgroup's flag
 
 // LDS carve-up, in floats
-constexpr int LDS_RED = 0;                                // [waves][4][64] partial tiles
-constexpr int LDS_STAT = LDS_RED + DS_WAVES * 4 * kWave;  // [2][waves][16 rows]
+constexpr int LDS_STAT = 0;                               // [2][waves][16 rows]
 constexpr int LDS_SMALL = LDS_STAT + 2 * DS_WAVES * 16;   // [2][waves]: attention max / sum per wave
 constexpr int LDS_BAD = LDS_SMALL + 2 * DS_WAVES;         // one int: a wait timed out
 constexpr int LDS_SINK = LDS_BAD + 32;                    // 1 KiB that prefetches write and nobody reads
-constexpr int LDS_FREE = LDS_SINK + 256;                  // attention scores | lm-head activations
+// GEMM phases: partial tiles [waves][NQ][64] | gamma, beta [2C]; attention: scores | partial
+// outputs; lm-head: normalised rows | gamma, beta
+constexpr int LDS_FREE = LDS_SINK + 256;
 
 
 // ---- cache-bypassing accesses for data that other workgroups wrote in this launch ---------
-__device__ __forceinline__ f32x4 load_bypass4(const float* p) {
-  f32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
-  return v;  // not valid before wait_vm() + pin()
-}
-// The same into a register that already holds a value: lanes that are switched off keep it.
-__device__ __forceinline__ void load_bypass4_into(f32x4& v, const float* p) {
-  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "+v"(v) : "v"(p) : "memory");
-}
-__device__ __forceinline__ void store_bypass4(float* p, f32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(p), "v"(v) : "memory");
-}
+// 128-bit ones go through buffer instructions, whose builtins take the cache policy (sc0 sc1)
+// and leave the bookkeeping of loads in flight to the compiler.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kBypass = 0x11;  // sc0 | sc1
+struct Bypass {
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ __forceinline__ Bypass(const float* base, size_t floats)
+      : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)(floats * sizeof(float)),
+                                               0x00020000)) {}
+  // float_index: this lane's first float (reads past `floats` return zero)
+  __device__ __forceinline__ f32x4 load4(int float_index) const {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, float_index * 4, 0, kBypass));
+  }
+  __device__ __forceinline__ void store4(int float_index, f32x4 v) const {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, float_index * 4, 0, kBypass);
+  }
+};
 __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
-// Makes later uses of v depend on this point of the instruction stream (after wait_vm()).
-__device__ __forceinline__ void pin(f32x4& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ float load_bypass(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -112,11 +117,23 @@ __device__ __forceinline__ void grid_arrive(const DecodeStep& a, unsigned epoch)
 __device__ __forceinline__ bool grid_wait(const DecodeStep& a, float* lds, unsigned epoch) {
   int* const bad = reinterpret_cast<int*>(lds + LDS_BAD);
   unsigned* const err = a.flags + (size_t)gridDim.x * FLAG_STRIDE;
-  for (int g = threadIdx.x; g < (int)gridDim.x; g += DS_THREADS) {
-    const unsigned* f = a.flags + (size_t)g * FLAG_STRIDE;
+  // Wave 0 polls, four flags per lane with all four loads in flight; it issues no prefetch, so
+  // nothing queues in front of its polls (loads return in order).  The other waves were sent
+  // off prefetching and come straight to the barrier below.
+  if (threadIdx.x < kWave) {
+    constexpr int PER = DS_GRID / kWave;
     unsigned spins = 0;
-    while ((int)(__hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - epoch) < 0) {
-      __builtin_amdgcn_s_sleep(1);
+    for (;;) {
+      unsigned v[PER];
+#pragma unroll
+      for (int i = 0; i < PER; i++)
+        v[i] = __hip_atomic_load(a.flags + (size_t)(threadIdx.x + kWave * i) * FLAG_STRIDE, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+      bool all = true;
+#pragma unroll
+      for (int i = 0; i < PER; i++) all = all && (int)(v[i] - epoch) >= 0;
+      if (all) break;
+      __builtin_amdgcn_s_sleep(2);
       ++spins;
       if (spins > a.spin_limit ||
           ((spins & 63) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
@@ -131,16 +148,6 @@ __device__ __forceinline__ bool grid_wait(const DecodeStep& a, float* lds, unsig
   return *bad == 0;
 }
 
-// A workgroup's share of the N output columns.
-struct Rows {
-  int n0, nrows;
-};
-__device__ __forceinline__ Rows wg_rows(int N) {
-  const int rp = (N + (int)gridDim.x - 1) / (int)gridDim.x;
-  const int n0 = (int)blockIdx.x * rp;
-  return {n0, min(rp, N - n0)};
-}
-
 // Warming the L2 of this workgroup's XCD with what the workgroup reads in its next phase:
 // loads that write to a scrap KiB of LDS (global_load_lds_dwordx4: no destination registers
 // that a late-landing load could clobber).  Issued right after the workgroup has arrived at
@@ -151,28 +158,31 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 __device__ __forceinline__ void touch(const float* p, float* lds) {
   __builtin_amdgcn_global_load_lds((glb_void_t*)p, (lds_void_t*)(lds + LDS_SINK), 16, 0, 0);
 }
-// n floats from p, 1 KiB per wave instruction, spread over the waves.
+constexpr int DS_PF_WAVES = DS_WAVES - 1;  // waves 1.. prefetch while wave 0 polls the barrier flags
+// n floats from p, 1 KiB per wave instruction, spread over the prefetching waves.
 __device__ __forceinline__ void prefetch_span(float* lds, const float* p, int n, int pw, int lane) {
-  for (int i = pw * 256 + lane * 4; i < n; i += DS_WAVES * 256) touch(p + i, lds);
+  for (int i = pw * 256 + lane * 4; i < n; i += DS_PF_WAVES * 256) touch(p + i, lds);
 }
 // The weight rows, bias and layernorm parameters of a GEMM phase.
 __device__ __forceinline__ void prefetch_gemm(float* lds, const float* W, const float* bias, int N, int K,
                                               const float* ln_w, const float* ln_b) {
   const int tid = opaque_tid(), lane = tid & 63;
-  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const Rows r = wg_rows(N);
-  if (r.nrows <= 0) return;
-  const float* wp = W + (size_t)(r.n0 + min(lane & 15, r.nrows - 1)) * K + 4 * (lane >> 4);
-  const int units = K >> 4;
-  for (int u = pw; u < units; u += DS_WAVES) touch(wp + (size_t)u * 16, lds);
+  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6) - 1;
+  if (pw < 0) return;
+  const int nrows = N / DS_GRID, n0 = (int)blockIdx.x * nrows;
+  // one instruction covers 4 rows x 256 bytes, as the phase's own loads do
+  for (int rg = 0; 4 * rg < nrows; rg++) {
+    const float* wp = W + (size_t)(n0 + min(4 * rg + (lane & 3), nrows - 1)) * K + 4 * (lane >> 2);
+    for (int u = pw; 64 * u < K; u += DS_PF_WAVES) touch(wp + (size_t)u * 64, lds);
+  }
   if (ln_w != nullptr) {
     prefetch_span(lds, ln_w, K, pw, lane);
     prefetch_span(lds, ln_b, K, pw, lane);
   }
   if (bias != nullptr && pw == 0 && lane < 5) {
     // the 16-byte pieces that hold bias[n0 .. n0 + nrows): at most five
-    const float* b0 = bias + ((r.n0 & ~3) + 4 * lane);
-    if (b0 < bias + r.n0 + r.nrows) touch(b0, lds);
+    const float* b0 = bias + ((n0 & ~3) + 4 * lane);
+    if (b0 < bias + n0 + nrows) touch(b0, lds);
   }
 }
 // The cache rows attention_item() will read for this workgroup's first (sequence, head): up to
@@ -180,14 +190,14 @@ __device__ __forceinline__ void prefetch_gemm(float* lds, const float* W, const 
 __device__ __forceinline__ void prefetch_cache(const DecodeStep& a, float* lds, const float* kc,
                                                const float* vc) {
   const int tid = opaque_tid(), lane = tid & 63;
-  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6) - 1;
   const int item = blockIdx.x;
-  if (item >= a.B * a.NH || a.pos < 1) return;
+  if (pw < 0 || item >= a.B * a.NH || a.pos < 1) return;
   const int b = item / a.NH, head = item % a.NH;
   const size_t off = (size_t)b * a.maxT * a.C + head * 64 + 4 * (lane & 15);
   const int last = a.pos - 1;  // rows 0..pos-1 exist; row pos is written by the phase itself
   for (int i = 0; i < 24; i++) {
-    const int t0 = 4 * (pw + DS_WAVES * i);
+    const int t0 = 4 * (pw + DS_PF_WAVES * i);
     if (t0 > last) break;
     const size_t row = (size_t)min(t0 + (lane >> 4), last) * a.C;
     touch(kc + off + row, lds);
@@ -195,143 +205,198 @@ __device__ __forceinline__ void prefetch_cache(const DecodeStep& a, float* lds, 
   }
 }
 
-// out[j][n0 + i] = resid + act( LN(in)[j] . W[n0 + i] + bias ) for this workgroup's columns.
-// A wave's share of K is NCH chunks of U units; a chunk's loads are all issued at once.
-// (NCH > 1 only without LN, whose statistics need the wave's whole share in registers.)
+// out[j][n0 + i] = resid + act( LN(in)[j] . W[n0 + i] + bias ) for this workgroup's ROWS output
+// columns n0 = ROWS * blockIdx.x, on v_mfma_f32_4x4x1_16B_f32: sixteen independent 4x4 outer
+// products per instruction, block b of lanes 4b..4b+3.  Lane (b, r) feeds weight row 4*rg + r
+// and activation row 4*jg + r at the same k, so a block accumulates a 4x4 tile of
+// (rows of group rg) x (sequences of group jg) over the k it is given; the 16 blocks take 16
+// different k (element e of the lane's 16 bytes at k = 64*c + 4*b + e), the 4 waves a quarter
+// of K each.  Loads are dense -- one instruction brings 256 bytes of each of 4 rows, every
+// lane a distinct 16 bytes -- which is what bounds a phase: the compute unit's load path
+// moves 64 bytes per cycle whether or not lanes repeat each other's addresses.  (A 16x16x4
+// tile with 3 weight rows and 8 sequences in it spent 5 us of a 9 us phase issuing loads that
+// were mostly repeats, and 3 us in mostly empty MFMAs.)  The 64 partial tiles (16 blocks x 4
+// waves) are summed through LDS in a fixed order.
+// KG: groups of 64 k per wave (K = 256 * KG); JG: groups of 4 sequences.
 // GATHER: the input rows are wte[ids[j]] + wpe[pos] (the first phase of a step); workgroup 0
 // also stores them as the residual stream x.
-template <bool LN, bool GELU, bool GATHER, int U, int NCH>
+template <bool LN, bool GELU, bool GATHER, int ROWS, int KG, int JG>
 __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, const float* __restrict__ W,
-                                           const float* __restrict__ bias, int N, int K,
-                                           const float* in, const float* __restrict__ ln_w,
-                                           const float* __restrict__ ln_b, float* out,
-                                           const float* resid, unsigned ph = 0) {
-  static_assert(!LN || NCH == 1, "a normalised row is held whole");
+                                           const float* __restrict__ bias, const float* in,
+                                           const float* __restrict__ ln_w, const float* __restrict__ ln_b,
+                                           float* out, const float* resid) {
+  constexpr int RG = (ROWS + 3) / 4;
+  constexpr int NQ = RG * JG * 4;       // accumulator registers: (rg, jg, v)
+  constexpr int NIT = (NQ + 31) / 32;   // epilogue passes of 32 registers
+  constexpr int K = 256 * KG, N = ROWS * DS_GRID;
   const int tid = opaque_tid(), lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r16 = lane & 15, kq = lane >> 4;
-  const Rows r = wg_rows(N);
-  if (r.nrows <= 0) return;  // the whole workgroup
+  const int blk = lane >> 2, r4 = lane & 3;
+  const int n0 = (int)blockIdx.x * ROWS;
   const int B = a.B;
-  // epilogue element of this thread: column n0 + oi of row oj
-  const int oi = tid & 15, oj = tid >> 4;
-  const bool owner = oi < r.nrows && oj < B;
-  float rs = 0.f, bs = 0.f;
-  if (owner) {
-    if (resid != nullptr) rs = load_bypass(resid + (size_t)oj * N + r.n0 + oi);
-    if (bias != nullptr) bs = bias[r.n0 + oi];
+  float* const red = lds + LDS_FREE;             // [wave][NQ][64]
+  float* const gb = red + DS_WAVES * NQ * kWave;  // gamma [K] | beta [K], with LN only
+
+  // Epilogue role: threads 8q..8q+7 sum register q (+32 per pass) over blocks and waves; the
+  // first of them finishes the four outputs (row 4*rg + v, sequences 4*jg .. 4*jg+3).
+  const int eq = tid >> 3, esub = tid & 7;
+  float rs[NIT][4], bs[NIT];
+#pragma unroll
+  for (int it = 0; it < NIT; it++) {
+    const int q = eq + 32 * it, row = 4 * (q / (4 * JG)) + (q & 3), j0 = 4 * ((q >> 2) % JG);
+    bs[it] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) rs[it][j] = 0.f;
+    if (esub == 0 && q < NQ && row < ROWS) {
+      if (bias != nullptr) bs[it] = bias[n0 + row];
+      if (resid != nullptr) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (j0 + j < B) rs[it][j] = load_bypass(resid + (size_t)(j0 + j) * N + n0 + row);
+      }
+    }
   }
 
-  // this lane's first float of the wave's share of K
-  const size_t koff = (size_t)wave * (U * NCH * 16) + 4 * kq;
-  const float* wp = W + (size_t)(r.n0 + r16) * K + koff;
-  // Loads cost the compute unit's one load path 64 bytes per cycle whether or not lanes
-  // repeat each other's addresses, so lanes beyond the workgroup's weight rows / beyond the
-  // B activation rows are switched off (their operands are zero) instead of clamped, and
-  // the layernorm's gamma and beta, which every row shares, go through LDS.
-  float* const gb = lds + LDS_FREE;  // gamma [K] | beta [K]
+  // this lane's first float of the wave's quarter of K
+  const int koff = wave * (KG * 64) + 4 * blk;
+  // Rows past the workgroup's share / past the B sequences repeat the last valid one (they
+  // feed accumulator entries that are never stored).
+  f32x4 wv[KG][RG], xv[KG][JG];
+  const Bypass xin(GATHER ? a.x : in, (size_t)B * K);
+#pragma unroll
+  for (int rg = 0; rg < RG; rg++) {
+    const float* wp = W + (size_t)(n0 + min(4 * rg + r4, ROWS - 1)) * K + koff;
+#pragma unroll
+    for (int c = 0; c < KG; c++) wv[c][rg] = *reinterpret_cast<const f32x4*>(wp + c * 64);
+  }
+#pragma unroll
+  for (int jg = 0; jg < JG; jg++) {
+    const int bj = min(4 * jg + r4, B - 1);
+    if (GATHER) {
+      const int id = a.ids[bj];
+      const bool ok = (unsigned)id < (unsigned)a.V;
+      const float* tp = a.wte + (size_t)(ok ? id : 0) * K + koff;
+      const float* pp = a.wpe_row + koff;
+      const float qn = __builtin_nanf("");
+#pragma unroll
+      for (int c = 0; c < KG; c++) {
+        xv[c][jg] = *reinterpret_cast<const f32x4*>(tp + c * 64) + *reinterpret_cast<const f32x4*>(pp + c * 64);
+        if (!ok) xv[c][jg] = f32x4{qn, qn, qn, qn};
+        if (blockIdx.x == 0 && 4 * jg + r4 < B) xin.store4(bj * K + koff + c * 64, xv[c][jg]);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < KG; c++) xv[c][jg] = xin.load4(bj * K + koff + c * 64);
+    }
+  }
+
   if (LN) {
     for (int i = tid * 4; i < K; i += DS_THREADS * 4) {
       *reinterpret_cast<f32x4*>(gb + i) = *reinterpret_cast<const f32x4*>(ln_w + i);
       *reinterpret_cast<f32x4*>(gb + K + i) = *reinterpret_cast<const f32x4*>(ln_b + i);
     }
   }
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (LN) {
+    // statistics of sequence 4*jg + r4: its row is spread over the 16 blocks of all 4 waves
+    float* const stat = lds + LDS_STAT;
+    float mean[JG], rstd[JG];
 #pragma unroll
-  for (int ch = 0; ch < NCH; ch++) {
-    f32x4 wv[U], xv[U];
-#pragma unroll
-    for (int c = 0; c < U; c++) {
-      wv[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-      xv[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    if (r16 < r.nrows) {
-#pragma unroll
-      for (int c = 0; c < U; c++) wv[c] = *reinterpret_cast<const f32x4*>(wp + (ch * U + c) * 16);
-    }
-    if (GATHER) {
-      if (r16 < B) {
-        const int id = a.ids[r16];
-        const bool ok = (unsigned)id < (unsigned)a.V;
-        const float* tp = a.wte + (size_t)(ok ? id : 0) * K + koff;
-        const float* pp = a.wpe_row + koff;
-        const float q = __builtin_nanf("");
-#pragma unroll
-        for (int c = 0; c < U; c++) {
-          xv[c] = *reinterpret_cast<const f32x4*>(tp + c * 16) + *reinterpret_cast<const f32x4*>(pp + c * 16);
-          if (!ok) xv[c] = f32x4{q, q, q, q};
-          if (blockIdx.x == 0) store_bypass4(a.x + (size_t)r16 * K + koff + c * 16, xv[c]);
-        }
-      }
-    } else {
-      if (r16 < B) {
-        const float* xp = in + (size_t)r16 * K + koff;
-#pragma unroll
-        for (int c = 0; c < U; c++) load_bypass4_into(xv[c], xp + (ch * U + c) * 16);
-      }
-      if (ch == 0) trace_mark(a, ph, 2);
-      wait_vm();
-#pragma unroll
-      for (int c = 0; c < U; c++) pin(xv[c]);
-      if (ch == 0) trace_mark(a, ph, 3);
-    }
-
-    if (LN) {
-      // row r16's statistics: lanes r16 + 16*kq of all the waves hold the row between them
-      float* const stat = lds + LDS_STAT;
+    for (int jg = 0; jg < JG; jg++) {
       float sum = 0.f;
 #pragma unroll
-      for (int c = 0; c < U; c++) sum += (xv[c][0] + xv[c][1]) + (xv[c][2] + xv[c][3]);
+      for (int c = 0; c < KG; c++) sum += (xv[c][jg][0] + xv[c][jg][1]) + (xv[c][jg][2] + xv[c][jg][3]);
+      sum += __shfl_xor(sum, 4, 64);
+      sum += __shfl_xor(sum, 8, 64);
       sum += __shfl_xor(sum, 16, 64);
       sum += __shfl_xor(sum, 32, 64);
-      if (kq == 0) stat[wave * 16 + r16] = sum;
-      __syncthreads();
-      float mean = 0.f;
+      if (blk == 0) stat[wave * 16 + 4 * jg + r4] = sum;
+    }
+    __syncthreads();
 #pragma unroll
-      for (int w = 0; w < DS_WAVES; w++) mean += stat[w * 16 + r16];
-      mean /= (float)K;
+    for (int jg = 0; jg < JG; jg++) {
+      float m = 0.f;
+#pragma unroll
+      for (int w = 0; w < DS_WAVES; w++) m += stat[w * 16 + 4 * jg + r4];
+      mean[jg] = m / (float)K;
       float q = 0.f;
 #pragma unroll
-      for (int c = 0; c < U; c++) {
-        const f32x4 d = xv[c] - mean;
+      for (int c = 0; c < KG; c++) {
+        const f32x4 d = xv[c][jg] - mean[jg];
         q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
       }
+      q += __shfl_xor(q, 4, 64);
+      q += __shfl_xor(q, 8, 64);
       q += __shfl_xor(q, 16, 64);
       q += __shfl_xor(q, 32, 64);
-      if (kq == 0) stat[DS_WAVES * 16 + wave * 16 + r16] = q;
-      __syncthreads();
+      if (blk == 0) stat[DS_WAVES * 16 + wave * 16 + 4 * jg + r4] = q;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int jg = 0; jg < JG; jg++) {
       float var = 0.f;
 #pragma unroll
-      for (int w = 0; w < DS_WAVES; w++) var += stat[DS_WAVES * 16 + w * 16 + r16];
-      const float rstd = 1.0f / sqrtf(var / (float)K + 1e-5f);
-#pragma unroll
-      for (int c = 0; c < U; c++)
-        xv[c] = (xv[c] - mean) * rstd * *reinterpret_cast<const f32x4*>(gb + koff + c * 16) +
-                *reinterpret_cast<const f32x4*>(gb + K + koff + c * 16);
-      trace_mark(a, ph, 4);
+      for (int w = 0; w < DS_WAVES; w++) var += stat[DS_WAVES * 16 + w * 16 + 4 * jg + r4];
+      rstd[jg] = 1.0f / sqrtf(var / (float)K + 1e-5f);
     }
-
 #pragma unroll
-    for (int c = 0; c < U; c++) {
+    for (int c = 0; c < KG; c++) {
+      const f32x4 g = *reinterpret_cast<const f32x4*>(gb + koff + c * 64);
+      const f32x4 be = *reinterpret_cast<const f32x4*>(gb + K + koff + c * 64);
 #pragma unroll
-      for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[c][e], xv[c][e], acc, 0, 0, 0);
+      for (int jg = 0; jg < JG; jg++) xv[c][jg] = (xv[c][jg] - mean[jg]) * rstd[jg] * g + be;
     }
   }
-  trace_mark(a, ph, 5);
-  // lane l holds D[4*(l/16) + v][l % 16]: weight row (output column) 4*(l/16)+v, activation row l%16
-  float* const red = lds + LDS_RED;
+
+  f32x4 acc[RG][JG];
 #pragma unroll
-  for (int v = 0; v < 4; v++) red[(wave * 4 + v) * kWave + lane] = acc[v];
+  for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+    for (int jg = 0; jg < JG; jg++) acc[rg][jg] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < KG; c++)
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+      for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int jg = 0; jg < JG; jg++)
+          acc[rg][jg] = __builtin_amdgcn_mfma_f32_4x4x1f32(wv[c][rg][e], xv[c][jg][e], acc[rg][jg], 0, 0, 0);
+
+  // register v of lane (b, r) of acc[rg][jg]: weight row 4*rg + v, sequence 4*jg + r, block b's k
+#pragma unroll
+  for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+    for (int jg = 0; jg < JG; jg++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) red[(wave * NQ + (rg * JG + jg) * 4 + v) * kWave + lane] = acc[rg][jg][v];
   __syncthreads();
-  if (owner) {
-    const int v = oi & 3, l = (oi >> 2) * 16 + oj;
-    float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < DS_WAVES; w++) sum += red[(w * 4 + v) * kWave + l];
-    sum += bs;
-    if (GELU) sum = gelu_tanh(sum);
-    sum += rs;
-    store_bypass(out + (size_t)oj * N + r.n0 + oi, sum);
+  for (int it = 0; it < NIT; it++) {
+    const int q = eq + 32 * it;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (q < NQ) {
+#pragma unroll
+      for (int w = 0; w < DS_WAVES; w++)
+#pragma unroll
+        for (int bi = 0; bi < 2; bi++)
+          sum += *reinterpret_cast<const f32x4*>(red + (w * NQ + q) * kWave + (2 * esub + bi) * 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      sum[j] += __shfl_xor(sum[j], 1, 64);
+      sum[j] += __shfl_xor(sum[j], 2, 64);
+      sum[j] += __shfl_xor(sum[j], 4, 64);
+    }
+    const int row = 4 * (q / (4 * JG)) + (q & 3), j0 = 4 * ((q >> 2) % JG);
+    if (esub == 0 && q < NQ && row < ROWS) {
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (j0 + j < B) {
+          float val = sum[j] + bs[it];
+          if (GELU) val = gelu_tanh(val);
+          store_bypass(out + (size_t)(j0 + j) * N + n0 + row, val + rs[it][j]);
+        }
+    }
   }
 }
 
@@ -350,22 +415,16 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
   float* const part = sc + ((pos + 64) & ~63);
   float* const small = lds + LDS_SMALL;
   const float scale = 0.125f;
-  const float* qrow = a.qkv + (size_t)b * 3 * C + head * 64 + 4 * sub;
   float* const kb = kc + (size_t)b * a.maxT * C + head * 64 + 4 * sub;
   float* const vb = vc + (size_t)b * a.maxT * C + head * 64 + 4 * sub;
 
-  f32x4 q4 = load_bypass4(qrow);
+  const Bypass qkv(a.qkv, (size_t)a.B * 3 * C);
+  const int qi = b * 3 * C + head * 64 + 4 * sub;
+  const f32x4 q4 = qkv.load4(qi);
   if (tid < 16) {
-    f32x4 kn = load_bypass4(qrow + C);
-    f32x4 vn = load_bypass4(qrow + 2 * C);
-    wait_vm();
-    pin(kn);
-    pin(vn);
-    *reinterpret_cast<f32x4*>(kb + (size_t)pos * C) = kn;
-    *reinterpret_cast<f32x4*>(vb + (size_t)pos * C) = vn;
+    *reinterpret_cast<f32x4*>(kb + (size_t)pos * C) = qkv.load4(qi + C);
+    *reinterpret_cast<f32x4*>(vb + (size_t)pos * C) = qkv.load4(qi + 2 * C);
   }
-  wait_vm();
-  pin(q4);
   __syncthreads();  // the appended row is visible to the whole workgroup
 
   float mx = -INFINITY;
@@ -446,19 +505,23 @@ __device__ __forceinline__ int lm_head_first_group(int wave) {
 template <int UC>
 __device__ __forceinline__ void prefetch_lm_head(const DecodeStep& a, float* lds) {
   const int tid = opaque_tid(), lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6) - 1;
+  if (pw < 0) return;
   const int K = a.C;
-  prefetch_span(lds, a.lnfw, K, wave, lane);
-  prefetch_span(lds, a.lnfb, K, wave, lane);
-  const int cg = lm_head_first_group(wave);
-  if (cg * 16 >= a.V) return;
-  const float* wp = a.wte + (size_t)min(cg * 16 + (lane & 15), a.V - 1) * K + 4 * (lane >> 4);
+  prefetch_span(lds, a.lnfw, K, pw, lane);
+  prefetch_span(lds, a.lnfb, K, pw, lane);
+  // the first chunk of every wave's first group, the polling wave's included
+  for (int wave = pw; wave < DS_WAVES; wave += DS_PF_WAVES) {
+    const int cg = lm_head_first_group(wave == DS_PF_WAVES ? 0 : wave + 1);
+    if (cg * 16 >= a.V) continue;
+    const float* wp = a.wte + (size_t)min(cg * 16 + (lane & 15), a.V - 1) * K + 4 * (lane >> 4);
 #pragma unroll
-  for (int c = 0; c < UC; c++) touch(wp + c * 16, lds);
+    for (int c = 0; c < UC; c++) touch(wp + c * 16, lds);
+  }
 }
 
-// U1: units of K per wave in the layernorm (K = 64 * U1); UC: units per chunk of a wave's sweep
-// over K (a divisor of 4 * U1).
+// U1: units of K per wave in the layernorm (K = 64 * U1); UC = 2 * U1: units per chunk of a
+// wave's sweep over K.
 template <int U1, int UC>
 __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   const int tid = opaque_tid(), lane = tid & 63;
@@ -475,16 +538,12 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
       *reinterpret_cast<f32x4*>(gb + K + i) = *reinterpret_cast<const f32x4*>(a.lnfb + i);
     }
     f32x4 xv[U1];
+    {
+      const Bypass xin(a.x, (size_t)B * K);
+      const int xi = min(r16, B - 1) * K + (int)koff;
 #pragma unroll
-    for (int c = 0; c < U1; c++) xv[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (r16 < B) {
-      const float* xp = a.x + (size_t)r16 * K + koff;
-#pragma unroll
-      for (int c = 0; c < U1; c++) load_bypass4_into(xv[c], xp + c * 16);
+      for (int c = 0; c < U1; c++) xv[c] = xin.load4(xi + c * 16);
     }
-    wait_vm();
-#pragma unroll
-    for (int c = 0; c < U1; c++) pin(xv[c]);
     float* const stat = lds + LDS_STAT;
     float sum = 0.f;
 #pragma unroll
@@ -521,25 +580,44 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
     __syncthreads();
   }
 
-  constexpr int NCH = 4 * U1 / UC;
-  static_assert(NCH * UC == 4 * U1, "UC must divide the units of K");
+  // Every group is two chunks of UC units (UC = half the units of K).  One chunk is always in
+  // flight ahead of the MFMAs, across group boundaries too: while chunk 1 of a group is
+  // multiplied, chunk 0 of the wave's next group is already loading.
+  static_assert(2 * UC == 4 * U1, "a group is two chunks");
   const float* const xrow = xs + (size_t)min(r16, B - 1) * ldx + 4 * kq;
-  for (int cg = lm_head_first_group(wave); cg * 16 < V; cg += (int)gridDim.x * DS_WAVES) {
+  const int step = (int)gridDim.x * DS_WAVES;
+  int cg = lm_head_first_group(wave);
+  f32x4 wa[UC], wb[UC];
+  const float* wp = a.wte + (size_t)min(cg * 16 + r16, V - 1) * K + 4 * kq;
+  if (cg * 16 < V) {
+#pragma unroll
+    for (int c = 0; c < UC; c++)
+      wa[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)c * 16));
+  }
+  for (; cg * 16 < V; cg += step) {
     const int n0 = cg * 16;
-    const float* wp = a.wte + (size_t)min(n0 + r16, V - 1) * K + 4 * kq;
+#pragma unroll
+    for (int c = 0; c < UC; c++)
+      wb[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)(UC + c) * 16));
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-    for (int ch = 0; ch < NCH; ch++) {
-      f32x4 wv[UC];
+#pragma unroll
+    for (int c = 0; c < UC; c++) {
+      const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + c * 16);
+#pragma unroll
+      for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wa[c][e], xq[e], acc, 0, 0, 0);
+    }
+    // rows of the next group (clamped: past the end nothing is stored, and the loop ends)
+    wp = a.wte + (size_t)min(n0 + step * 16 + r16, V - 1) * K + 4 * kq;
+    if ((cg + step) * 16 < V) {
 #pragma unroll
       for (int c = 0; c < UC; c++)
-        wv[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)(ch * UC + c) * 16));
+        wa[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)c * 16));
+    }
 #pragma unroll
-      for (int c = 0; c < UC; c++) {
-        const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + (ch * UC + c) * 16);
+    for (int c = 0; c < UC; c++) {
+      const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + (UC + c) * 16);
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[c][e], xq[e], acc, 0, 0, 0);
-      }
+      for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wb[c][e], xq[e], acc, 0, 0, 0);
     }
     if (r16 < B) {
       float* op = a.logits + (size_t)r16 * V + n0 + 4 * kq;
@@ -550,14 +628,14 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   }
 }
 
-// U1: units of K (16 floats) per wave where K = C (C = 64 * U1, so every wave has exactly that
-// many and the loops carry no guards); where K = 4C a wave takes N4 chunks of U4 units
-// (U4 * N4 = 4 * U1).  ULM: units per chunk of the lm-head's sweep.
-template <int U1, int U4, int N4, int ULM>
+// KG1 = C / 256: groups of 64 k per wave where K = C, and weight rows per workgroup where
+// N = C (the grid is exactly DS_GRID = 256 workgroups).  JG: groups of 4 sequences.
+// ULM: units of 16 k per chunk of the lm-head's sweep.
+template <int KG1, int JG, int ULM>
 __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeStep a) {
   extern __shared__ float lds[];
-  const int C = a.C;
-  const size_t cs = (size_t)C;
+  constexpr int C = 256 * KG1;
+  constexpr size_t cs = (size_t)C;
   unsigned* const err = a.flags + (size_t)gridDim.x * FLAG_STRIDE;
   // a launch that follows a failed one does nothing until the host has cleared the error
   if (threadIdx.x == 0)
@@ -571,11 +649,11 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
   for (int l = 0; l < a.L; l++) {
     // qkv = LN1(x) Wqkv + b
     if (l == 0)
-      gemm_phase<true, false, true, U1, 1>(a, lds, a.qkvw, a.qkvb, 3 * C, C, nullptr, a.ln1w, a.ln1b,
-                                               a.qkv, nullptr, epoch - a.epoch0);
+      gemm_phase<true, false, true, 3 * KG1, KG1, JG>(a, lds, a.qkvw, a.qkvb, nullptr, a.ln1w, a.ln1b, a.qkv,
+                                                      nullptr);
     else
-      gemm_phase<true, false, false, U1, 1>(a, lds, a.qkvw + l * 3 * cs * cs, a.qkvb + l * 3 * cs, 3 * C,
-                                                C, a.x, a.ln1w + l * cs, a.ln1b + l * cs, a.qkv, nullptr, epoch - a.epoch0);
+      gemm_phase<true, false, false, 3 * KG1, KG1, JG>(a, lds, a.qkvw + l * 3 * cs * cs, a.qkvb + l * 3 * cs,
+                                                       a.x, a.ln1w + l * cs, a.ln1b + l * cs, a.qkv, nullptr);
     grid_arrive(a, ++epoch);
     prefetch_cache(a, lds, a.kv + (2 * (size_t)l) * a.plane, a.kv + (2 * (size_t)l + 1) * a.plane);
     if (!grid_wait(a, lds, epoch)) return;
@@ -589,22 +667,22 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += y Wproj + b
-    gemm_phase<false, false, false, U1, 1>(a, lds, a.attprojw + l * cs * cs, a.attprojb + l * cs, C, C,
-                                               a.atty, nullptr, nullptr, a.x, a.x, epoch - a.epoch0);
+    gemm_phase<false, false, false, KG1, KG1, JG>(a, lds, a.attprojw + l * cs * cs, a.attprojb + l * cs, a.atty,
+                                                  nullptr, nullptr, a.x, a.x);
     grid_arrive(a, ++epoch);
     prefetch_gemm(lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, 4 * C, C, a.ln2w + l * cs, a.ln2b + l * cs);
     if (!grid_wait(a, lds, epoch)) return;
 
     // h = gelu(LN2(x) Wfc + b)
-    gemm_phase<true, true, false, U1, 1>(a, lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, 4 * C, C,
-                                             a.x, a.ln2w + l * cs, a.ln2b + l * cs, a.h, nullptr, epoch - a.epoch0);
+    gemm_phase<true, true, false, 4 * KG1, KG1, JG>(a, lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, a.x,
+                                                    a.ln2w + l * cs, a.ln2b + l * cs, a.h, nullptr);
     grid_arrive(a, ++epoch);
     prefetch_gemm(lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, C, 4 * C, nullptr, nullptr);
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += h Wfcproj + b
-    gemm_phase<false, false, false, U4, N4>(a, lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, C,
-                                               4 * C, a.h, nullptr, nullptr, a.x, a.x, epoch - a.epoch0);
+    gemm_phase<false, false, false, KG1, 4 * KG1, JG>(a, lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs,
+                                                      a.h, nullptr, nullptr, a.x, a.x);
     grid_arrive(a, ++epoch);
     if (l + 1 < a.L)
       prefetch_gemm(lds, a.qkvw + (l + 1) * 3 * cs * cs, a.qkvb + (l + 1) * 3 * cs, 3 * C, C,
@@ -613,64 +691,77 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
       prefetch_lm_head<ULM>(a, lds);
     if (!grid_wait(a, lds, epoch)) return;
   }
-  lm_head_phase<U1, ULM>(a, lds);
+  lm_head_phase<4 * KG1, ULM>(a, lds);
   trace_mark(a, 5u * (unsigned)a.L, 0);
 }
 
 // ---- host ---------------------------------------------------------------------------------
-int decode_step_workgroups(int device) {
+// The kernel runs on exactly DS_GRID workgroups, one per compute unit, all resident at once.
+static bool device_has_grid(int device) {
   static int cached_device = -1, cached = 0;
-  if (device == cached_device) return cached;
-  int cus = 0;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
-  cached_device = device;
-  cached = cus;
-  return cus;
+  if (device != cached_device) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return false;
+    cached_device = device;
+    cached = cus;
+  }
+  return cached >= DS_GRID;
 }
 
 size_t decode_step_flag_bytes(int device) {
-  return ((size_t)decode_step_workgroups(device) * FLAG_STRIDE + FLAG_STRIDE) * sizeof(unsigned);
+  (void)device;
+  return ((size_t)DS_GRID * FLAG_STRIDE + FLAG_STRIDE) * sizeof(unsigned);
+}
+
+size_t decode_step_probe_slots(int num_layers) {
+  return (size_t)DS_GRID * TRACE_SLOTS * (5 * (size_t)num_layers + 1);
 }
 
 static size_t decode_step_lds_bytes(const GPT2Config& c, int B, int pos) {
-  const size_t att = (size_t)((pos + 64) & ~63) + DS_WAVES * 64;
-  const size_t lm = (size_t)B * (c.channels + 4) + 2 * (size_t)c.channels;  // rows | gamma | beta
-  return (LDS_FREE + (att > lm ? att : lm)) * sizeof(float);
+  const size_t C = c.channels, jg = (B + 3) / 4;
+  const size_t gemm = 2 * C + DS_WAVES * ((C / 256) * jg * 4) * kWave;  // gamma, beta | partial tiles
+  const size_t att = (size_t)((pos + 64) & ~63) + DS_WAVES * 64;        // scores | partial outputs
+  const size_t lm = (size_t)B * (C + 4) + 2 * C;                        // rows | gamma, beta
+  size_t most = gemm > att ? gemm : att;
+  if (lm > most) most = lm;
+  return (LDS_FREE + most) * sizeof(float);
 }
 
 bool decode_step_supported(const GPT2Config& c, int B, int device) {
-  const int C = c.channels, G = decode_step_workgroups(device);
-  if (G < 1 || G > DS_THREADS) return false;
+  const int C = c.channels;
+  if (!device_has_grid(device)) return false;
   if (B < 1 || B > 16 || c.num_heads * 64 != C) return false;
-  // every wave takes exactly C/64 (4C/64) units of 16 floats of K; instantiated sizes only
-  if (C != 64 && C != 128 && C != 256 && C != 512 && C != 768 && C != 1024) return false;
-  if ((4 * C + G - 1) / G > 16) return false;  // the widest N: at most 16 weight rows per workgroup
+  if (C != 256 && C != 512 && C != 768 && C != 1024) return false;  // the instantiated sizes
   return decode_step_lds_bytes(c, B, c.max_seq_len - 1) <= 160 * 1024;
 }
 
-int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) {
-  const int G = decode_step_workgroups(device);
-  const size_t lds = decode_step_lds_bytes(c, step.B, step.pos);
-  const void* kernel;
-  int slot;
-  switch (c.channels) {
-    case 64: kernel = reinterpret_cast<const void*>(decode_step_kernel<1, 4, 1, 4>); slot = 0; break;
-    case 128: kernel = reinterpret_cast<const void*>(decode_step_kernel<2, 8, 1, 8>); slot = 1; break;
-    case 256: kernel = reinterpret_cast<const void*>(decode_step_kernel<4, 16, 1, 16>); slot = 2; break;
-    case 512: kernel = reinterpret_cast<const void*>(decode_step_kernel<8, 32, 1, 16>); slot = 3; break;
-    case 768: kernel = reinterpret_cast<const void*>(decode_step_kernel<12, 48, 1, 24>); slot = 4; break;
-    case 1024: kernel = reinterpret_cast<const void*>(decode_step_kernel<16, 32, 2, 32>); slot = 5; break;
-    default: return fail(GPT2HIP_EINVAL, "decode step kernel: channels %d not supported", c.channels);
+template <int KG1, int ULM>
+static const void* kernel_for(int jg) {
+  switch (jg) {
+    case 1: return reinterpret_cast<const void*>(decode_step_kernel<KG1, 1, ULM>);
+    case 2: return reinterpret_cast<const void*>(decode_step_kernel<KG1, 2, ULM>);
+    case 3: return reinterpret_cast<const void*>(decode_step_kernel<KG1, 3, ULM>);
+    default: return reinterpret_cast<const void*>(decode_step_kernel<KG1, 4, ULM>);
   }
-  static bool lds_raised[6] = {false, false, false, false, false, false};
-  if (lds > 48 * 1024 && !lds_raised[slot]) {
+}
+
+int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) {
+  if (!decode_step_supported(c, step.B, device))
+    return fail(GPT2HIP_EINVAL, "decode step kernel: model or batch not supported");
+  const size_t lds = decode_step_lds_bytes(c, step.B, step.pos);
+  const int jg = (step.B + 3) / 4, kg1 = c.channels / 256;
+  const void* kernel = kg1 == 1   ? kernel_for<1, 8>(jg)
+                       : kg1 == 2 ? kernel_for<2, 16>(jg)
+                       : kg1 == 3 ? kernel_for<3, 24>(jg)
+                                  : kernel_for<4, 32>(jg);
+  static bool lds_raised[4][4] = {};
+  if (lds > 48 * 1024 && !lds_raised[kg1 - 1][jg - 1]) {
     G2_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    lds_raised[slot] = true;
+    lds_raised[kg1 - 1][jg - 1] = true;
   }
   DecodeStep copy = step;
   void* args[] = {&copy};
-  G2_HIP(hipLaunchCooperativeKernel(kernel, dim3((unsigned)G), dim3(DS_THREADS), args, (unsigned)lds,
-                                    stream()));
+  G2_HIP(hipLaunchCooperativeKernel(kernel, dim3(DS_GRID), dim3(DS_THREADS), args, (unsigned)lds, stream()));
   return GPT2HIP_OK;
 }
 

@@ -532,9 +532,7 @@ size_t gpt2_decode_probe_size(const GPT2* model) {
   if (!model || !model->step_persistent || model->kv_batch < 1 ||
       !decode_step_supported(model->cfg, model->kv_batch, model->device))
     return 0;
-  // the flag array holds one 64-byte line per workgroup and one for the error word
-  const size_t workgroups = decode_step_flag_bytes(model->device) / (16 * sizeof(unsigned)) - 1;
-  return workgroups * (8 * (5 * (size_t)model->cfg.num_layers + 1));
+  return decode_step_probe_slots(model->cfg.num_layers);
 }
 
 namespace g2 {

@@ -16,8 +16,8 @@ LOGIT_TOL = 2e-3
 
 @pytest.mark.parametrize("cfg,B,T0,steps", [
     (dict(max_seq_len=48, vocab_size=211, num_layers=2, num_heads=4, channels=256), 3, 5, 6),
-    (dict(max_seq_len=16, vocab_size=50, num_layers=1, num_heads=1, channels=64), 2, 3, 3),
-    (dict(max_seq_len=80, vocab_size=331, num_layers=3, num_heads=2, channels=128), 5, 37, 4),
+    (dict(max_seq_len=300, vocab_size=1031, num_layers=2, num_heads=8, channels=512), 5, 7, 3),
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=4, channels=256), 13, 37, 3),
     (dict(max_seq_len=128, vocab_size=3001, num_layers=2, num_heads=16, channels=1024), 4, 100, 3),
     (dict(max_seq_len=300, vocab_size=1031, num_layers=3, num_heads=8, channels=512), 16, 250, 5),
     (dict(max_seq_len=64, vocab_size=50257, num_layers=2, num_heads=12, channels=768), 1, 1, 4),
