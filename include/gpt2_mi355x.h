@@ -202,8 +202,8 @@ int gpt2_prefill_status(GPT2* model, const int* inputs_device, int B, int T);
 int gpt2_decode_status(GPT2* model, const int* next_ids_device);
 /* How gpt2_decode runs (no counterpart in the reference).  persistent != 0 (the default): one
  * persistent kernel per step where it takes the model (up to 16 sequences, head size 64,
- * channels <= 768 and a multiple of 16), otherwise one launch per operation; 0: always one
- * launch per operation.  spin_limit bounds the polls a workgroup of the persistent kernel
+ * channels 256, 512, 768 or 1024, a device with at least 256 compute units), otherwise one
+ * launch per operation; 0: always one launch per operation.  spin_limit bounds the polls a workgroup of the persistent kernel
  * spends on one flag of its grid barrier before it gives up and ends the kernel (default
  * 2^21); a step that gave up makes the NEXT gpt2_decode call fail and empties the cache. */
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit);

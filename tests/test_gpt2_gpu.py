@@ -270,6 +270,109 @@ def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
         model.close()
 
 
+@pytest.mark.parametrize("cfg,B,T0,steps", [
+    (dict(max_seq_len=48, vocab_size=211, num_layers=2, num_heads=4, channels=256), 3, 5, 6),
+    (dict(max_seq_len=300, vocab_size=1031, num_layers=2, num_heads=8, channels=512), 5, 7, 3),
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=4, channels=256), 13, 37, 3),
+    (dict(max_seq_len=128, vocab_size=3001, num_layers=2, num_heads=16, channels=1024), 4, 100, 3),
+    (dict(max_seq_len=300, vocab_size=1031, num_layers=3, num_heads=8, channels=512), 16, 250, 5),
+    (dict(max_seq_len=64, vocab_size=50257, num_layers=2, num_heads=12, channels=768), 1, 1, 4),
+    (dict(g2.GPT2_124M), 8, 120, 10),
+])
+def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_path(cfg, B, T0, steps):
+    print(f"persistent decode cfg={cfg} B={B} T0={T0} steps={steps}", flush=True)
+    params = syn.make_params(91, perturb_affine=True, **cfg)
+    ids = syn.make_tokens(92, B, T0 + steps, cfg["vocab_size"])
+    exp_logits, _, _ = oracle.gpt2_forward(params, ids, maxT=cfg["max_seq_len"], V=cfg["vocab_size"],
+                                           L=cfg["num_layers"], NH=cfg["num_heads"],
+                                           C=cfg["channels"], want_lnf=True)
+    dids = torch.from_numpy(ids).cuda()
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(params)
+        runs = {}
+        for persistent in (False, True):
+            model.decode_options(persistent=persistent)
+            model.prefill(dids[:, :T0].contiguous())
+            out = []
+            for s in range(steps):
+                print(f"  persistent={persistent} step {s}", flush=True)
+                out.append(model.decode(dids[:, T0 + s].contiguous()).cpu().numpy())
+            runs[persistent] = np.stack(out)
+            assert model.cache_length() == T0 + steps
+        for s in range(steps):
+            d = np.abs(runs[True][s] - exp_logits[:, T0 + s]).max()
+            dd = np.abs(runs[True][s] - runs[False][s]).max()
+            print(f"  step {s}: max|dlogits| vs oracle {d:.3e}, vs per-launch path {dd:.3e}", flush=True)
+            assert np.isfinite(runs[True][s]).all()
+            assert d <= LOGIT_TOL
+            assert np.array_equal(runs[True][s].argmax(-1), exp_logits[:, T0 + s].argmax(-1))
+    finally:
+        model.close()
+
+def test_gpt2_persistent_decode_gives_up_a_barrier_wait_cleanly():
+    """Failure handling of the persistent kernel's grid barrier, forced from the host: with a
+    spin limit of 0 the first workgroup that has to wait gives up, every workgroup leaves the
+    kernel, a later call reports it, and the model works again after a new prompt."""
+    cfg = dict(max_seq_len=32, vocab_size=211, num_layers=2, num_heads=4, channels=256)
+    params = syn.make_params(93, perturb_affine=True, **cfg)
+    ids = torch.from_numpy(syn.make_tokens(94, 2, 8, cfg["vocab_size"])).cuda()
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(params)
+        model.decode_options(persistent=False)
+        model.prefill(ids[:, :7].contiguous())
+        want = model.decode(ids[:, 7].contiguous()).clone()
+        model.decode_options(persistent=True, spin_limit=0)
+        model.prefill(ids[:, :7].contiguous())
+        print("  step with spin limit 0", flush=True)
+        model.decode(ids[:, 7].contiguous())       # launches; some workgroup gives up
+        torch.cuda.synchronize()                   # the kernel has ended by itself
+        with pytest.raises(g2.GPT2HipError, match="grid barrier"):
+            model.decode(ids[:, 7].contiguous())
+        assert model.cache_length() == 0
+        model.decode_options(persistent=True)
+        model.prefill(ids[:, :7].contiguous())
+        got = model.decode(ids[:, 7].contiguous())
+        torch.cuda.synchronize()
+        assert (got - want).abs().max().item() <= 1e-4
+    finally:
+        model.close()
+
+
+def test_gpt2_decode_probe_clocks_are_ordered():
+    cfg = dict(max_seq_len=32, vocab_size=211, num_layers=2, num_heads=4, channels=256)
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(syn.make_params(95, **cfg))
+        ids = torch.from_numpy(syn.make_tokens(96, 3, 6, cfg["vocab_size"])).cuda()
+        model.prefill(ids[:, :5].contiguous())
+        ref = model.decode(ids[:, 5].contiguous()).clone()
+        model.prefill(ids[:, :5].contiguous())
+        clk = model.decode_probe(ids[:, 5].contiguous()).cpu().numpy()
+        torch.cuda.synchronize()
+        assert torch.equal(model.step_logits(), ref)           # the probe changes no result
+        phases = 5 * cfg["num_layers"] + 1
+        assert clk.shape[:2] == (phases, 2)
+        done, passed = clk[:, 0, :], clk[:-1, 1, :]
+        assert (done > 0).all() and (passed > 0).all()
+        assert (passed >= done[:-1]).all()                      # a barrier is passed after arriving
+        assert (passed.min(axis=1) >= done[:-1].max(axis=1)).all()   # ... and after EVERYBODY arrived
+        assert (done[1:] >= passed).all()
+        # a model the persistent kernel does not take
+        small = g2.GPT2(max_seq_len=16, vocab_size=50, num_layers=1, num_heads=1, channels=64)
+        try:
+            small.load_params(syn.make_params(97, max_seq_len=16, vocab_size=50, num_layers=1, num_heads=1,
+                                              channels=64))
+            small.prefill(torch.zeros(1, 3, dtype=torch.int32, device="cuda"))
+            with pytest.raises(g2.GPT2HipError):
+                small.decode_probe(torch.zeros(1, dtype=torch.int32, device="cuda"))
+        finally:
+            small.close()
+    finally:
+        model.close()
+
+
 def test_gpt2_decode_error_paths():
     cfg = dict(max_seq_len=8, vocab_size=50, num_layers=1, num_heads=1, channels=64)
     model = g2.GPT2(**cfg)
