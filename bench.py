@@ -288,57 +288,57 @@ def clock_probe(g2):
 
 def decode_bench(model, cfg, B, T0, steps):
     """Incremental inference: a prompt of T0 tokens per sequence, then `steps` single-token
-    steps against the key/value cache.  A step is bound by streaming the weights (and the
-    cache rows read by attention) from HBM once."""
+    steps against the key/value cache, once with one launch per operation and once with the
+    persistent decode-step kernel.  A step is bound by streaming the weights (and the cache
+    rows read by attention) from HBM once: that is the roofline the GB/s figure is set against."""
     import torch
     V, C, L = cfg["vocab_size"], cfg["channels"], cfg["num_layers"]
     ids = torch.randint(0, V, (B, T0), dtype=torch.int32, device="cuda")
     nxt = torch.randint(0, V, (steps + 4, B), dtype=torch.int32, device="cuda")
-    model.prefill(ids)
-    for i in range(4):
-        model.decode(nxt[i])
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    model.prefill(ids)
-    torch.cuda.synchronize()
-    prefill_ms = (time.perf_counter() - t0) * 1e3
-    t0 = time.perf_counter()
-    for i in range(steps):
-        model.decode(nxt[4 + i])
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / steps * 1e3
     pos = T0 + steps / 2
     weight_bytes = 4 * (L * (12 * C * C + 13 * C) + V * C + 2 * C)
     cache_bytes = 2 * L * B * pos * C * 4
-    gbs = (weight_bytes + cache_bytes) / ms / 1e6
-    row = {"decode": f"B={B}, prompt T0={T0}, {steps} steps", "prefill_ms": prefill_ms,
-           "ms_per_step": ms, "tokens_per_s": B / ms * 1e3,
-           "bytes_per_step": weight_bytes + cache_bytes, "GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
-           "finite": bool(torch.isfinite(model.step_logits()).all())}
+    out = {"decode": f"B={B}, prompt T0={T0}, {steps} steps", "bytes_per_step": weight_bytes + cache_bytes}
+    for name, persistent in (("launch_per_operation", False), ("persistent_kernel", True)):
+        model.decode_options(persistent=persistent)
+        model.prefill(ids)
+        for i in range(4):
+            model.decode(nxt[i])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.prefill(ids)
+        torch.cuda.synchronize()
+        out["prefill_ms"] = (time.perf_counter() - t0) * 1e3
+        t0 = time.perf_counter()
+        for i in range(steps):
+            model.decode(nxt[4 + i])
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        gbs = (weight_bytes + cache_bytes) / ms / 1e6
+        out[name] = {"ms_per_step": ms, "tokens_per_s": B / ms * 1e3, "GB/s": gbs,
+                     "frac_hbm": gbs / PEAK_HBM_GBS,
+                     "finite": bool(torch.isfinite(model.step_logits()).all())}
     try:
         # one more step with the persistent kernel's clock probe: per phase kind, the mean time
         # a workgroup works and the mean time from its arrival to everybody's arrival
         clk = model.decode_probe(nxt[0]).cpu().numpy().astype("float64") * 10.0  # ns
         names = ("qkv", "attention", "attproj", "fc_gelu", "fcproj")
         done, passed = clk[:, 0, :], clk[:, 1, :]
-        start = clk[0, 0, :].min()
         work = {n: [] for n in names}
         wait = {n: [] for n in names}
-        prev = None
         for p in range(5 * L):
-            begin = passed[p - 1] if p else None
-            if begin is not None:
-                work[names[p % 5]].append(float((done[p] - begin).mean()))
+            if p:
+                work[names[p % 5]].append(float((done[p] - passed[p - 1]).mean()))
             wait[names[p % 5]].append(float((passed[p] - done[p]).mean()))
-        row["probe_us"] = {
-            "kernel": float((done[5 * L].max() - start) / 1e3),
+        out["persistent_kernel"]["probe_us"] = {
+            "kernel": float((done[5 * L].max() - clk[0, 0, :].min()) / 1e3),
             "lm_head": float((done[5 * L] - passed[5 * L - 1]).mean() / 1e3),
             "work": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in work.items()},
             "barrier": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in wait.items()}}
     except g2.GPT2HipError:
-        pass
-    log("  decode", json.dumps(row))
-    return row
+        out["persistent_kernel"]["note"] = "the persistent kernel does not take this model or batch"
+    log("  decode", json.dumps(out))
+    return out
 
 
 def cpu_baseline(model, cfg, B, T):
@@ -495,6 +495,8 @@ def main():
         result["standalone"] = standalone(g2)
         for r in result["standalone"]:
             log("  standalone", json.dumps(r))
+        # the path's next caller: incremental decoding against a key/value cache
+        result["decode"] = decode_bench(model, cfg, B, 128, 64)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(model, cfg, B, T)
         log("  cpu_baseline", json.dumps(result["cpu_baseline"]))
