@@ -407,6 +407,7 @@ def main():
     model.reserve(B, T)
     if args.decode:
         print(json.dumps({"decode": [decode_bench(model, cfg, B, T, args.decode)]}))
+        model.close()
         return
 
     for _ in range(args.warmup):

@@ -759,9 +759,13 @@ int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) 
     G2_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     lds_raised[kg1 - 1][jg - 1] = true;
   }
+  // An ordinary launch: with one workgroup per compute unit's worth of resources and nothing
+  // else running on the device, all DS_GRID workgroups are resident at once, which the grid
+  // barrier needs.  If they ever are not (a device shared with other work), the barrier's
+  // bounded wait ends the kernel and the error is reported; it cannot hang.
   DecodeStep copy = step;
   void* args[] = {&copy};
-  G2_HIP(hipLaunchCooperativeKernel(kernel, dim3(DS_GRID), dim3(DS_THREADS), args, (unsigned)lds, stream()));
+  G2_HIP(hipLaunchKernel(kernel, dim3(DS_GRID), dim3(DS_THREADS), args, lds, stream()));
   return GPT2HIP_OK;
 }
 
