@@ -424,6 +424,18 @@ def main():
     log(f"forward {args.model} B={B} T={T}: {ms_per_step:.3f} ms/step, {tokens_per_s:,.0f} tok/s"
         f" (logits finite: {finite})")
 
+    # the llm.c signature: token ids handed over in host memory (32 KiB per step here), copied
+    # in stream order and waited for before the launches are issued; not the reported value
+    host_ids = ids.cpu().numpy()
+    model.forward(host_ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.forward(host_ids)
+    torch.cuda.synchronize()
+    host_ids_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    log(f"  with host token ids (gpt2_forward): {host_ids_ms:.3f} ms/step")
+
     graph_ms = None
     if args.graph:
         for _ in range(max(args.warmup, 2)):          # the first call captures
@@ -490,6 +502,7 @@ def main():
         "forward_frac_fp32_mfma": (sum(flops.values()) / (ms_per_step * 1e9)) / PEAK_FP32_MFMA_TFLOPS,
         "kernels": kernels,
     }
+    result["host_ids_ms_per_step"] = host_ids_ms
     if graph_ms is not None:
         result["graph_replay_ms_per_step"] = graph_ms
     if not args.no_standalone:
