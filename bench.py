@@ -514,6 +514,26 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(model, cfg, B, T)
         log("  cpu_baseline", json.dumps(result["cpu_baseline"]))
+    if not args.no_standalone and args.model == "124M" and B == 8 and T == 1024:
+        # the second end-to-end workload: GPT-2 350M, B=4, T=1024
+        model.close()
+        cfg2 = dict(g2.GPT2_350M)
+        model = g2.GPT2(**cfg2)
+        init_params_on_device(model, syn, cfg2, seed=1338)
+        ids2 = torch.randint(0, cfg2["vocab_size"], (4, 1024), dtype=torch.int32, device="cuda")
+        for _ in range(args.warmup):
+            model.forward(ids2)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            model.forward(ids2)
+        torch.cuda.synchronize()
+        ms2 = (time.perf_counter() - t0) / args.steps * 1e3
+        fl2 = sum(forward_flops(cfg2, 4, 1024).values())
+        result["gpt2_350M_B4_T1024"] = {
+            "ms_per_step": ms2, "tokens_per_s": 4 * 1024 / ms2 * 1e3,
+            "forward_frac_fp32_mfma": fl2 / (ms2 * 1e9) / PEAK_FP32_MFMA_TFLOPS}
+        log("  350M", json.dumps(result["gpt2_350M_B4_T1024"]))
     model.close()
     print(json.dumps(result), flush=True)
 

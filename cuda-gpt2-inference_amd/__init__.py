@@ -68,7 +68,23 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err)
+    build_example()
     return LIB_PATH
+
+
+EXAMPLE_SRC = os.path.join(_HERE, "examples", "llmc_style_driver.cpp")
+EXAMPLE_BIN = os.path.join(_HERE, "examples", "llmc_style_driver")
+
+
+def build_example() -> str:
+    """Compile the plain-C++ llm.c-style driver against the library's C ABI (host code only)."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "-O2", "-std=c++17", EXAMPLE_SRC, "-I", os.path.join(_ROOT, "include"),
+           "-L", _HERE, "-lgpt2_mi355x", "-Wl,-rpath,$ORIGIN/..", "-o", EXAMPLE_BIN]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on the example driver ({proc.returncode}):\n{proc.stderr}")
+    return EXAMPLE_BIN
 
 
 class GPT2Config(ctypes.Structure):

@@ -1,0 +1,141 @@
+// What an llm.c-style driver looks like against the C ABI of libgpt2_mi355x.so, in the
+// reference's own host language: plain C++ that owns its device buffers (hipMalloc) and calls
+// the launchers layer by layer with llm.c's argument lists -- the call sequence of llm.c's
+// gpt2_forward with the reference's two fusions (reference README.md:9-19,255-268;
+// kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:237-246).  The same model is then run
+// through the library's own gpt2_forward driver, and the two sets of logits must be equal bit
+// for bit: they are the same kernels in the same order.  Exit status 0 on agreement.
+//
+//   hipcc llmc_style_driver.cpp -I<repo>/include -L<repo>/cuda-gpt2-inference_amd \
+//         -lgpt2_mi355x -Wl,-rpath,<repo>/cuda-gpt2-inference_amd -o llmc_style_driver
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "gpt2_mi355x.h"
+
+#define HIP_OK(expr)                                                                  \
+  do {                                                                                \
+    hipError_t e_ = (expr);                                                           \
+    if (e_ != hipSuccess) {                                                           \
+      fprintf(stderr, "%s: %s (%s:%d)\n", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+      exit(2);                                                                        \
+    }                                                                                 \
+  } while (0)
+
+// Seeded N(0, sigma) from a 64-bit LCG and Box-Muller: any fixed parameters will do here.
+struct Rng {
+  uint64_t s;
+  double uniform() {
+    s = s * 6364136223846793005ULL + 1442695040888963407ULL;
+    return ((s >> 11) + 0.5) / 9007199254740992.0;
+  }
+  float normal(float sigma) {
+    const double u = uniform(), v = uniform();
+    return sigma * (float)(std::sqrt(-2.0 * std::log(u)) * std::cos(6.283185307179586 * v));
+  }
+};
+
+int main(int argc, char** argv) {
+  // a small GPT-2: sizes chosen to exercise edge tiles (V and T are not multiples of a tile)
+  const int maxT = 96, V = 1031, L = 3, NH = 4, C = 256, B = 3, T = 77;
+  const size_t c = C;
+  (void)argc;
+  (void)argv;
+
+  // parameters in llm.c checkpoint order
+  const size_t sizes[16] = {(size_t)V * c, (size_t)maxT * c, L * c,     L * c, L * 3 * c * c, L * 3 * c,
+                            L * c * c,     L * c,            L * c,     L * c, L * 4 * c * c, L * 4 * c,
+                            L * c * 4 * c, L * c,            c,         c};
+  size_t off[17] = {0};
+  for (int i = 0; i < 16; i++) off[i + 1] = off[i] + sizes[i];
+  std::vector<float> hp(off[16]);
+  Rng rng{20240326};
+  for (int i = 0; i < 16; i++) {
+    const bool gamma = (i == 2 || i == 8 || i == 14);
+    const float sigma = (i == 1) ? 0.01f : 0.02f;
+    for (size_t j = 0; j < sizes[i]; j++) hp[off[i] + j] = (gamma ? 1.0f : 0.0f) + rng.normal(gamma ? 0.1f : sigma);
+  }
+  std::vector<int> hids((size_t)B * T);
+  for (auto& id : hids) id = (int)(rng.uniform() * V) % V;
+
+  // ---- the llm.c way: the driver owns parameters and activations -------------------------
+  float* params;
+  HIP_OK(hipMalloc((void**)&params, hp.size() * sizeof(float)));
+  HIP_OK(hipMemcpy(params, hp.data(), hp.size() * sizeof(float), hipMemcpyHostToDevice));
+  const float *wte = params + off[0], *wpe = params + off[1], *ln1w = params + off[2], *ln1b = params + off[3],
+              *qkvw = params + off[4], *qkvb = params + off[5], *attprojw = params + off[6],
+              *attprojb = params + off[7], *ln2w = params + off[8], *ln2b = params + off[9],
+              *fcw = params + off[10], *fcb = params + off[11], *fcprojw = params + off[12],
+              *fcprojb = params + off[13], *lnfw = params + off[14], *lnfb = params + off[15];
+  const size_t M = (size_t)B * T;
+  int* ids;
+  float *res_a, *res_b, *ln, *qkv, *atty, *proj, *fch, *logits, *mean, *rstd;
+  HIP_OK(hipMalloc((void**)&ids, M * sizeof(int)));
+  HIP_OK(hipMalloc((void**)&res_a, M * c * 4));
+  HIP_OK(hipMalloc((void**)&res_b, M * c * 4));
+  HIP_OK(hipMalloc((void**)&ln, M * c * 4));
+  HIP_OK(hipMalloc((void**)&qkv, M * 3 * c * 4));
+  HIP_OK(hipMalloc((void**)&atty, M * c * 4));
+  HIP_OK(hipMalloc((void**)&proj, M * c * 4));
+  HIP_OK(hipMalloc((void**)&fch, M * 4 * c * 4));
+  HIP_OK(hipMalloc((void**)&logits, M * V * 4));
+  HIP_OK(hipMalloc((void**)&mean, M * 4));
+  HIP_OK(hipMalloc((void**)&rstd, M * 4));
+  HIP_OK(hipMemcpy(ids, hids.data(), M * sizeof(int), hipMemcpyHostToDevice));
+
+  float *residual = res_a, *other = res_b;
+  encoder_forward(residual, ids, wte, wpe, B, T, C);
+  layernorm_forward(ln, mean, rstd, residual, ln1w, ln1b, B, T, C);
+  for (int l = 0; l < L; l++) {
+    matmul_forward(qkv, ln, qkvw + l * 3 * c * c, qkvb + l * 3 * c, B, T, C, 3 * C);
+    attention_forward(atty, /*qkvr=*/nullptr, /*att=*/nullptr, qkv, B, T, C, NH);
+    matmul_forward(proj, atty, attprojw + l * c * c, attprojb + l * c, B, T, C, C);
+    fused_residual_layernorm_forward(other, ln, mean, rstd, residual, proj, ln2w + l * c, ln2b + l * c, B, T, C);
+    matmul_forward_gelu(fch, ln, fcw + l * 4 * c * c, fcb + l * 4 * c, B, T, C, 4 * C, /*is_gelu=*/1);
+    matmul_forward(proj, fch, fcprojw + l * 4 * c * c, fcprojb + l * c, B, T, 4 * C, C);
+    const float* nw = (l + 1 < L) ? ln1w + (l + 1) * c : lnfw;
+    const float* nb = (l + 1 < L) ? ln1b + (l + 1) * c : lnfb;
+    fused_residual_layernorm_forward(residual, ln, mean, rstd, other, proj, nw, nb, B, T, C);
+  }
+  matmul_forward(logits, ln, wte, /*bias=*/nullptr, B, T, C, V);
+  HIP_OK(hipDeviceSynchronize());
+  std::vector<float> mine(M * V);
+  HIP_OK(hipMemcpy(mine.data(), logits, mine.size() * 4, hipMemcpyDeviceToHost));
+
+  // ---- the library's own driver on the same parameters and tokens ------------------------
+  GPT2Config cfg = {maxT, V, L, NH, C};
+  GPT2* model = gpt2_create(&cfg);
+  if (!model || gpt2_load_params_host(model, hp.data(), hp.size()) != GPT2HIP_OK) {
+    fprintf(stderr, "gpt2_create / gpt2_load_params_host: %s\n", gpt2hip_last_error());
+    return 2;
+  }
+  gpt2_forward(model, hids.data(), B, T);
+  HIP_OK(hipDeviceSynchronize());
+  std::vector<float> theirs(M * V);
+  HIP_OK(hipMemcpy(theirs.data(), gpt2_logits(model), theirs.size() * 4, hipMemcpyDeviceToHost));
+
+  // an error is an error code, not an abort, through the _status forms
+  const int rc = matmul_forward_status(logits, ln, wte, nullptr, B, T, /*C=*/0, V);
+  const bool reports = rc == GPT2HIP_EINVAL && std::strlen(gpt2hip_last_error()) > 0;
+
+  double sum = 0.0, maxdiff = 0.0;
+  bool finite = true;
+  for (size_t i = 0; i < mine.size(); i++) {
+    finite = finite && std::isfinite(mine[i]);
+    sum += mine[i];
+    maxdiff = std::fmax(maxdiff, std::fabs((double)mine[i] - (double)theirs[i]));
+  }
+  printf("llmc_style_driver: L=%d C=%d B=%d T=%d V=%d: sum(logits)=%.6f max|launchers - gpt2_forward|=%g "
+         "finite=%d status_form_reports=%d\n", L, C, B, T, V, sum, maxdiff, (int)finite, (int)reports);
+
+  gpt2_destroy(model);
+  void* bufs[] = {params, ids, res_a, res_b, ln, qkv, atty, proj, fch, logits, mean, rstd};
+  for (void* p : bufs) HIP_OK(hipFree(p));
+  return (finite && maxdiff == 0.0 && reports) ? 0 : 1;
+}

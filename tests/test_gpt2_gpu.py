@@ -5,6 +5,7 @@ different fp32 summation orders can only differ where the oracle's top-2 gap is
 itself at rounding level, so a mismatch is reported together with that gap.
 """
 import importlib
+import os
 import sys
 
 import numpy as np
@@ -371,6 +372,19 @@ def test_gpt2_decode_probe_clocks_are_ordered():
             small.close()
     finally:
         model.close()
+
+
+def test_cpp_driver_calling_the_launchers_equals_gpt2_forward():
+    """The plain-C++ llm.c-style driver (examples/llmc_style_driver.cpp, built by build()): its
+    layer-by-layer launcher calls must give the logits of the library's own gpt2_forward bit
+    for bit, and the _status forms must report errors instead of aborting."""
+    import subprocess
+    assert os.path.exists(g2.EXAMPLE_BIN), "build() compiles the example driver"
+    print("running", g2.EXAMPLE_BIN, flush=True)
+    proc = subprocess.run([g2.EXAMPLE_BIN], capture_output=True, text=True, timeout=100)
+    print(proc.stdout, proc.stderr, flush=True)
+    assert proc.returncode == 0
+    assert "max|launchers - gpt2_forward|=0 " in proc.stdout
 
 
 def test_gpt2_decode_error_paths():
