@@ -82,6 +82,14 @@ def test_gpt2_350M_B1_T128():
     check(*run_both(dict(g2.GPT2_350M), 1, 128, seed=21))
 
 
+@pytest.mark.parametrize("C,NH", [(1280, 20), (1600, 25)])
+def test_gpt2_wider_models_one_layer(C, NH):
+    # the widths of GPT-2 large and XL (one block of each): K and N the 124M / 350M shapes do
+    # not exercise (1280, 3840, 5120, 1600, 4800, 6400), 20 and 25 heads
+    cfg = dict(max_seq_len=1024, vocab_size=50257, num_layers=1, num_heads=NH, channels=C)
+    check(*run_both(cfg, 2, 200, seed=51, perturb=True))
+
+
 @pytest.mark.parametrize("name,B,T", [("124M", 8, 1024), ("350M", 4, 1024)])
 def test_gpt2_full_size_against_the_oracle(name, B, T):
     """The benchmark's own workloads, whole: every logit of the (B*T, V) result against the
