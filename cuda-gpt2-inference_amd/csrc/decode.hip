@@ -53,10 +53,9 @@ constexpr int FLAG_STRIDE = 16;  // one 64-byte line per workgroup's flag
 constexpr int LDS_STAT = 0;                               // [2][waves][16 rows]
 constexpr int LDS_SMALL = LDS_STAT + 2 * DS_WAVES * 16;   // [2][waves]: attention max / sum per wave
 constexpr int LDS_BAD = LDS_SMALL + 2 * DS_WAVES;         // one int: a wait timed out
-constexpr int LDS_SINK = LDS_BAD + 32;                    // 1 KiB that prefetches write and nobody reads
 // GEMM phases: partial tiles [waves][NQ][64] | gamma, beta [2C]; attention: scores | partial
 // outputs; lm-head: normalised rows | gamma, beta
-constexpr int LDS_FREE = LDS_SINK + 256;
+constexpr int LDS_FREE = LDS_BAD + 32;
 
 
 // ---- cache-bypassing accesses for data that other workgroups wrote in this launch ---------
@@ -117,9 +116,8 @@ __device__ __forceinline__ void grid_arrive(const DecodeStep& a, unsigned epoch)
 __device__ __forceinline__ bool grid_wait(const DecodeStep& a, float* lds, unsigned epoch) {
   int* const bad = reinterpret_cast<int*>(lds + LDS_BAD);
   unsigned* const err = a.flags + (size_t)gridDim.x * FLAG_STRIDE;
-  // Wave 0 polls, four flags per lane with all four loads in flight; it issues no prefetch, so
-  // nothing queues in front of its polls (loads return in order).  The other waves were sent
-  // off prefetching and come straight to the barrier below.
+  // Wave 0 polls, four flags per lane with all four loads in flight; the other waves come
+  // straight to the barrier below.
   if (threadIdx.x < kWave) {
     constexpr int PER = DS_GRID / kWave;
     unsigned spins = 0;
@@ -148,60 +146,51 @@ __device__ __forceinline__ bool grid_wait(const DecodeStep& a, float* lds, unsig
   return *bad == 0;
 }
 
-// Warming the L2 of this workgroup's XCD with what the workgroup reads in its next phase:
-// loads that write to a scrap KiB of LDS (global_load_lds_dwordx4: no destination registers
-// that a late-landing load could clobber).  Issued right after the workgroup has arrived at
-// a grid barrier, so that HBM latency runs while the barrier is waited for; the phase's own
-// loads then hit the L2.
-typedef __attribute__((address_space(3))) void lds_void_t;
-typedef const __attribute__((address_space(1))) void glb_void_t;
-__device__ __forceinline__ void touch(const float* p, float* lds) {
-  __builtin_amdgcn_global_load_lds((glb_void_t*)p, (lds_void_t*)(lds + LDS_SINK), 16, 0, 0);
-}
-constexpr int DS_PF_WAVES = DS_WAVES - 1;  // waves 1.. prefetch while wave 0 polls the barrier flags
-// n floats from p, 1 KiB per wave instruction, spread over the prefetching waves.
-__device__ __forceinline__ void prefetch_span(float* lds, const float* p, int n, int pw, int lane) {
-  for (int i = pw * 256 + lane * 4; i < n; i += DS_PF_WAVES * 256) touch(p + i, lds);
-}
-// The weight rows, bias and layernorm parameters of a GEMM phase.
-__device__ __forceinline__ void prefetch_gemm(float* lds, const float* W, const float* bias, int N, int K,
-                                              const float* ln_w, const float* ln_b) {
+// What a GEMM phase needs that does not depend on other workgroups: this lane's pieces of
+// the workgroup's ROWS weight rows, this thread's piece of gamma and beta, the bias of the
+// outputs this thread finishes.  It is loaded into registers one phase AHEAD, while the
+// previous phase computes: HBM latency (and the 7-9 MB burst the 256 workgroups make of it)
+// then runs under that phase's arithmetic, not in front of this phase and not while a grid
+// barrier's flags have to get through the memory system.
+template <int ROWS, int KG, int JG, bool LN>
+struct PhaseWeights {
+  static constexpr int RG = (ROWS + 3) / 4;
+  static constexpr int NQ = RG * JG * 4;       // accumulator registers: (rg, jg, v)
+  static constexpr int NIT = (NQ + 31) / 32;   // epilogue passes of 32 registers
+  static constexpr int K = 256 * KG;
+  f32x4 w[KG][RG];
+  f32x4 g, b;       // gamma / beta [4 * tid .. 4 * tid + 3]
+  float bias[NIT];  // of output row 4*rg + v, for the thread that finishes register q = (rg, jg, v)
+};
+template <int ROWS, int KG, int JG, bool LN>
+__device__ __forceinline__ void load_phase_weights(PhaseWeights<ROWS, KG, JG, LN>& pw, const float* __restrict__ W,
+                                                   const float* __restrict__ bias,
+                                                   const float* __restrict__ ln_w,
+                                                   const float* __restrict__ ln_b) {
+  using PW = PhaseWeights<ROWS, KG, JG, LN>;
   const int tid = opaque_tid(), lane = tid & 63;
-  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6) - 1;
-  if (pw < 0) return;
-  const int nrows = N / DS_GRID, n0 = (int)blockIdx.x * nrows;
-  // one instruction covers 4 rows x 256 bytes, as the phase's own loads do
-  for (int rg = 0; 4 * rg < nrows; rg++) {
-    const float* wp = W + (size_t)(n0 + min(4 * rg + (lane & 3), nrows - 1)) * K + 4 * (lane >> 2);
-    for (int u = pw; 64 * u < K; u += DS_PF_WAVES) touch(wp + (size_t)u * 64, lds);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int blk = lane >> 2, r4 = lane & 3;
+  const int n0 = (int)blockIdx.x * ROWS;
+  const int koff = wave * (KG * 64) + 4 * blk;  // this lane's first float of the wave's quarter of K
+  // rows past the workgroup's share repeat the last one (they feed accumulator entries that
+  // are never stored)
+#pragma unroll
+  for (int rg = 0; rg < PW::RG; rg++) {
+    const float* wp = W + (size_t)(n0 + min(4 * rg + r4, ROWS - 1)) * PW::K + koff;
+#pragma unroll
+    for (int c = 0; c < KG; c++) pw.w[c][rg] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + c * 64));
   }
-  if (ln_w != nullptr) {
-    prefetch_span(lds, ln_w, K, pw, lane);
-    prefetch_span(lds, ln_b, K, pw, lane);
+  if (LN) {
+    const int i = min(4 * tid, PW::K - 4);
+    pw.g = *reinterpret_cast<const f32x4*>(ln_w + i);
+    pw.b = *reinterpret_cast<const f32x4*>(ln_b + i);
   }
-  if (bias != nullptr && pw == 0 && lane < 5) {
-    // the 16-byte pieces that hold bias[n0 .. n0 + nrows): at most five
-    const float* b0 = bias + ((n0 & ~3) + 4 * lane);
-    if (b0 < bias + n0 + nrows) touch(b0, lds);
-  }
-}
-// The cache rows attention_item() will read for this workgroup's first (sequence, head): up to
-// 24 wave instructions (4 rows of 256 bytes each) of keys and as many of values per wave.
-__device__ __forceinline__ void prefetch_cache(const DecodeStep& a, float* lds, const float* kc,
-                                               const float* vc) {
-  const int tid = opaque_tid(), lane = tid & 63;
-  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6) - 1;
-  const int item = blockIdx.x;
-  if (pw < 0 || item >= a.B * a.NH || a.pos < 1) return;
-  const int b = item / a.NH, head = item % a.NH;
-  const size_t off = (size_t)b * a.maxT * a.C + head * 64 + 4 * (lane & 15);
-  const int last = a.pos - 1;  // rows 0..pos-1 exist; row pos is written by the phase itself
-  for (int i = 0; i < 24; i++) {
-    const int t0 = 4 * (pw + DS_PF_WAVES * i);
-    if (t0 > last) break;
-    const size_t row = (size_t)min(t0 + (lane >> 4), last) * a.C;
-    touch(kc + off + row, lds);
-    touch(vc + off + row, lds);
+  const int eq = tid >> 3;
+#pragma unroll
+  for (int it = 0; it < PW::NIT; it++) {
+    const int q = eq + 32 * it, row = 4 * (q / (4 * JG)) + (q & 3);
+    pw.bias[it] = bias[n0 + min(row, ROWS - 1)];
   }
 }
 
@@ -220,14 +209,12 @@ __device__ __forceinline__ void prefetch_cache(const DecodeStep& a, float* lds, 
 // KG: groups of 64 k per wave (K = 256 * KG); JG: groups of 4 sequences.
 // GATHER: the input rows are wte[ids[j]] + wpe[pos] (the first phase of a step); workgroup 0
 // also stores them as the residual stream x.
-template <bool LN, bool GELU, bool GATHER, int ROWS, int KG, int JG>
-__device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, const float* __restrict__ W,
-                                           const float* __restrict__ bias, const float* in,
-                                           const float* __restrict__ ln_w, const float* __restrict__ ln_b,
-                                           float* out, const float* resid) {
-  constexpr int RG = (ROWS + 3) / 4;
-  constexpr int NQ = RG * JG * 4;       // accumulator registers: (rg, jg, v)
-  constexpr int NIT = (NQ + 31) / 32;   // epilogue passes of 32 registers
+template <bool LN, bool GELU, bool GATHER, int ROWS, int KG, int JG, typename LoadNext>
+__device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
+                                           const PhaseWeights<ROWS, KG, JG, LN>& pw, const float* in, float* out,
+                                           const float* resid, LoadNext&& load_next) {
+  using PW = PhaseWeights<ROWS, KG, JG, LN>;
+  constexpr int RG = PW::RG, NQ = PW::NQ, NIT = PW::NIT;
   constexpr int K = 256 * KG, N = ROWS * DS_GRID;
   const int tid = opaque_tid(), lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -240,15 +227,13 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
   // Epilogue role: threads 8q..8q+7 sum register q (+32 per pass) over blocks and waves; the
   // first of them finishes the four outputs (row 4*rg + v, sequences 4*jg .. 4*jg+3).
   const int eq = tid >> 3, esub = tid & 7;
-  float rs[NIT][4], bs[NIT];
+  float rs[NIT][4];
 #pragma unroll
   for (int it = 0; it < NIT; it++) {
     const int q = eq + 32 * it, row = 4 * (q / (4 * JG)) + (q & 3), j0 = 4 * ((q >> 2) % JG);
-    bs[it] = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; j++) rs[it][j] = 0.f;
     if (esub == 0 && q < NQ && row < ROWS) {
-      if (bias != nullptr) bs[it] = bias[n0 + row];
       if (resid != nullptr) {
 #pragma unroll
         for (int j = 0; j < 4; j++)
@@ -259,16 +244,9 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
 
   // this lane's first float of the wave's quarter of K
   const int koff = wave * (KG * 64) + 4 * blk;
-  // Rows past the workgroup's share / past the B sequences repeat the last valid one (they
-  // feed accumulator entries that are never stored).
-  f32x4 wv[KG][RG], xv[KG][JG];
+  // Sequences past B repeat the last one (they feed accumulator entries that are never stored).
+  f32x4 xv[KG][JG];
   const Bypass xin(GATHER ? a.x : in, (size_t)B * K);
-#pragma unroll
-  for (int rg = 0; rg < RG; rg++) {
-    const float* wp = W + (size_t)(n0 + min(4 * rg + r4, ROWS - 1)) * K + koff;
-#pragma unroll
-    for (int c = 0; c < KG; c++) wv[c][rg] = *reinterpret_cast<const f32x4*>(wp + c * 64);
-  }
 #pragma unroll
   for (int jg = 0; jg < JG; jg++) {
     const int bj = min(4 * jg + r4, B - 1);
@@ -290,12 +268,14 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
     }
   }
 
-  if (LN) {
-    for (int i = tid * 4; i < K; i += DS_THREADS * 4) {
-      *reinterpret_cast<f32x4*>(gb + i) = *reinterpret_cast<const f32x4*>(ln_w + i);
-      *reinterpret_cast<f32x4*>(gb + K + i) = *reinterpret_cast<const f32x4*>(ln_b + i);
-    }
+  if (LN && 4 * tid < K) {
+    *reinterpret_cast<f32x4*>(gb + 4 * tid) = pw.g;
+    *reinterpret_cast<f32x4*>(gb + K + 4 * tid) = pw.b;
   }
+  // The activations of this phase have arrived (so has everything requested earlier): the
+  // next phase's weights are requested now and arrive under this phase's arithmetic.
+  wait_vm();
+  load_next();
   if (LN) {
     // statistics of sequence 4*jg + r4: its row is spread over the 16 blocks of all 4 waves
     float* const stat = lds + LDS_STAT;
@@ -311,7 +291,7 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
       sum += __shfl_xor(sum, 32, 64);
       if (blk == 0) stat[wave * 16 + 4 * jg + r4] = sum;
     }
-    __syncthreads();
+    lds_barrier();  // not __syncthreads(): that would wait for the next phase's weights in flight
 #pragma unroll
     for (int jg = 0; jg < JG; jg++) {
       float m = 0.f;
@@ -330,7 +310,7 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
       q += __shfl_xor(q, 32, 64);
       if (blk == 0) stat[DS_WAVES * 16 + wave * 16 + 4 * jg + r4] = q;
     }
-    __syncthreads();
+    lds_barrier();  // not __syncthreads(): that would wait for the next phase's weights in flight
 #pragma unroll
     for (int jg = 0; jg < JG; jg++) {
       float var = 0.f;
@@ -360,7 +340,7 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
       for (int rg = 0; rg < RG; rg++)
 #pragma unroll
         for (int jg = 0; jg < JG; jg++)
-          acc[rg][jg] = __builtin_amdgcn_mfma_f32_4x4x1f32(wv[c][rg][e], xv[c][jg][e], acc[rg][jg], 0, 0, 0);
+          acc[rg][jg] = __builtin_amdgcn_mfma_f32_4x4x1f32(pw.w[c][rg][e], xv[c][jg][e], acc[rg][jg], 0, 0, 0);
 
   // register v of lane (b, r) of acc[rg][jg]: weight row 4*rg + v, sequence 4*jg + r, block b's k
 #pragma unroll
@@ -369,7 +349,7 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
     for (int jg = 0; jg < JG; jg++)
 #pragma unroll
       for (int v = 0; v < 4; v++) red[(wave * NQ + (rg * JG + jg) * 4 + v) * kWave + lane] = acc[rg][jg][v];
-  __syncthreads();
+  lds_barrier();  // not __syncthreads(): that would wait for the next phase's weights in flight
 #pragma unroll
   for (int it = 0; it < NIT; it++) {
     const int q = eq + 32 * it;
@@ -392,7 +372,7 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds, cons
 #pragma unroll
       for (int j = 0; j < 4; j++)
         if (j0 + j < B) {
-          float val = sum[j] + bs[it];
+          float val = sum[j] + pw.bias[it];
           if (GELU) val = gelu_tanh(val);
           store_bypass(out + (size_t)(j0 + j) * N + n0 + row, val + rs[it][j]);
         }
@@ -498,30 +478,12 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
 
 // logits = LNf(x) . wte^T.  The normalised rows go to LDS once per workgroup; wave w then
 // takes the 16-row groups g + gridDim.x * (w + 4 i) of wte for the whole K, UC units at a
-// time; the first units of its first group were requested into the L2 before the last barrier.
+// time.
 __device__ __forceinline__ int lm_head_first_group(int wave) {
   return (int)blockIdx.x + (int)gridDim.x * wave;
 }
-template <int UC>
-__device__ __forceinline__ void prefetch_lm_head(const DecodeStep& a, float* lds) {
-  const int tid = opaque_tid(), lane = tid & 63;
-  const int pw = __builtin_amdgcn_readfirstlane(tid >> 6) - 1;
-  if (pw < 0) return;
-  const int K = a.C;
-  prefetch_span(lds, a.lnfw, K, pw, lane);
-  prefetch_span(lds, a.lnfb, K, pw, lane);
-  // the first chunk of every wave's first group, the polling wave's included
-  for (int wave = pw; wave < DS_WAVES; wave += DS_PF_WAVES) {
-    const int cg = lm_head_first_group(wave == DS_PF_WAVES ? 0 : wave + 1);
-    if (cg * 16 >= a.V) continue;
-    const float* wp = a.wte + (size_t)min(cg * 16 + (lane & 15), a.V - 1) * K + 4 * (lane >> 4);
-#pragma unroll
-    for (int c = 0; c < UC; c++) touch(wp + c * 16, lds);
-  }
-}
-
-// U1: units of K per wave in the layernorm (K = 64 * U1); UC = 2 * U1: units per chunk of a
-// wave's sweep over K.
+// U1: units of K per wave in the layernorm (K = 64 * U1); UC: units per chunk of a wave's
+// sweep over K.
 template <int U1, int UC>
 __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   const int tid = opaque_tid(), lane = tid & 63;
@@ -580,10 +542,11 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
     __syncthreads();
   }
 
-  // Every group is two chunks of UC units (UC = half the units of K).  One chunk is always in
-  // flight ahead of the MFMAs, across group boundaries too: while chunk 1 of a group is
-  // multiplied, chunk 0 of the wave's next group is already loading.
-  static_assert(2 * UC == 4 * U1, "a group is two chunks");
+  // Every group is NCH (even) chunks of UC units.  One chunk is always in flight ahead of the
+  // MFMAs, across group boundaries too: while the last chunk of a group is multiplied, the
+  // first chunk of the wave's next group is already loading.
+  constexpr int NCH = 4 * U1 / UC;
+  static_assert(NCH * UC == 4 * U1 && NCH % 2 == 0, "a group is an even number of chunks");
   const float* const xrow = xs + (size_t)min(r16, B - 1) * ldx + 4 * kq;
   const int step = (int)gridDim.x * DS_WAVES;
   int cg = lm_head_first_group(wave);
@@ -596,29 +559,32 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   }
   for (; cg * 16 < V; cg += step) {
     const int n0 = cg * 16;
-#pragma unroll
-    for (int c = 0; c < UC; c++)
-      wb[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)(UC + c) * 16));
+    const float* const wnext = a.wte + (size_t)min(n0 + step * 16 + r16, V - 1) * K + 4 * kq;
+    const bool more = (cg + step) * 16 < V;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < UC; c++) {
-      const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + c * 16);
+    for (int ch = 0; ch < NCH; ch++) {
+      f32x4(&cur)[UC] = (ch & 1) ? wb : wa;
+      f32x4(&nxt)[UC] = (ch & 1) ? wa : wb;
+      if (ch + 1 < NCH) {
 #pragma unroll
-      for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wa[c][e], xq[e], acc, 0, 0, 0);
+        for (int c = 0; c < UC; c++)
+          nxt[c] = __builtin_nontemporal_load(
+              reinterpret_cast<const f32x4*>(wp + (size_t)((ch + 1) * UC + c) * 16));
+      } else if (more) {
+        // rows of the next group (clamped: past the end nothing is stored, and the loop ends)
+#pragma unroll
+        for (int c = 0; c < UC; c++)
+          nxt[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wnext + (size_t)c * 16));
+      }
+#pragma unroll
+      for (int c = 0; c < UC; c++) {
+        const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + (ch * UC + c) * 16);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(cur[c][e], xq[e], acc, 0, 0, 0);
+      }
     }
-    // rows of the next group (clamped: past the end nothing is stored, and the loop ends)
-    wp = a.wte + (size_t)min(n0 + step * 16 + r16, V - 1) * K + 4 * kq;
-    if ((cg + step) * 16 < V) {
-#pragma unroll
-      for (int c = 0; c < UC; c++)
-        wa[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)c * 16));
-    }
-#pragma unroll
-    for (int c = 0; c < UC; c++) {
-      const f32x4 xq = *reinterpret_cast<const f32x4*>(xrow + (UC + c) * 16);
-#pragma unroll
-      for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wb[c][e], xq[e], acc, 0, 0, 0);
-    }
+    wp = wnext;
     if (r16 < B) {
       float* op = a.logits + (size_t)r16 * V + n0 + 4 * kq;
 #pragma unroll
@@ -645,50 +611,52 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
   if (*reinterpret_cast<int*>(lds + LDS_BAD) != 0) return;
   unsigned epoch = a.epoch0;
 
+  const int items = a.B * a.NH;  // (sequence, head) pairs of the attention phase
+  PhaseWeights<3 * KG1, KG1, JG, true> w_qkv;
+  PhaseWeights<KG1, KG1, JG, false> w_proj;
+  PhaseWeights<4 * KG1, KG1, JG, true> w_fc;
+  PhaseWeights<KG1, 4 * KG1, JG, false> w_fcproj;
+  load_phase_weights(w_qkv, a.qkvw, a.qkvb, a.ln1w, a.ln1b);
 #pragma unroll 1
   for (int l = 0; l < a.L; l++) {
+    float* const kc = a.kv + (2 * (size_t)l) * a.plane;
+    float* const vc = kc + a.plane;
     // qkv = LN1(x) Wqkv + b
+    auto next_proj = [&]() { load_phase_weights(w_proj, a.attprojw + l * cs * cs, a.attprojb + l * cs, nullptr, nullptr); };
     if (l == 0)
-      gemm_phase<true, false, true, 3 * KG1, KG1, JG>(a, lds, a.qkvw, a.qkvb, nullptr, a.ln1w, a.ln1b, a.qkv,
-                                                      nullptr);
+      gemm_phase<true, false, true>(a, lds, w_qkv, nullptr, a.qkv, nullptr, next_proj);
     else
-      gemm_phase<true, false, false, 3 * KG1, KG1, JG>(a, lds, a.qkvw + l * 3 * cs * cs, a.qkvb + l * 3 * cs,
-                                                       a.x, a.ln1w + l * cs, a.ln1b + l * cs, a.qkv, nullptr);
+      gemm_phase<true, false, false>(a, lds, w_qkv, a.x, a.qkv, nullptr, next_proj);
     grid_arrive(a, ++epoch);
-    prefetch_cache(a, lds, a.kv + (2 * (size_t)l) * a.plane, a.kv + (2 * (size_t)l + 1) * a.plane);
     if (!grid_wait(a, lds, epoch)) return;
 
     // attention over the cache
-    for (int item = blockIdx.x; item < a.B * a.NH; item += gridDim.x)
-      attention_item(a, lds, a.kv + (2 * (size_t)l) * a.plane, a.kv + (2 * (size_t)l + 1) * a.plane,
-                     item / a.NH, item % a.NH);
+    for (int item = blockIdx.x; item < items; item += gridDim.x)
+      attention_item(a, lds, kc, vc, item / a.NH, item % a.NH);
     grid_arrive(a, ++epoch);
-    prefetch_gemm(lds, a.attprojw + l * cs * cs, a.attprojb + l * cs, C, C, nullptr, nullptr);
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += y Wproj + b
-    gemm_phase<false, false, false, KG1, KG1, JG>(a, lds, a.attprojw + l * cs * cs, a.attprojb + l * cs, a.atty,
-                                                  nullptr, nullptr, a.x, a.x);
+    gemm_phase<false, false, false>(a, lds, w_proj, a.atty, a.x, a.x, [&]() {
+      load_phase_weights(w_fc, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, a.ln2w + l * cs, a.ln2b + l * cs);
+    });
     grid_arrive(a, ++epoch);
-    prefetch_gemm(lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, 4 * C, C, a.ln2w + l * cs, a.ln2b + l * cs);
     if (!grid_wait(a, lds, epoch)) return;
 
     // h = gelu(LN2(x) Wfc + b)
-    gemm_phase<true, true, false, 4 * KG1, KG1, JG>(a, lds, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, a.x,
-                                                    a.ln2w + l * cs, a.ln2b + l * cs, a.h, nullptr);
+    gemm_phase<true, true, false>(a, lds, w_fc, a.x, a.h, nullptr, [&]() {
+      load_phase_weights(w_fcproj, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, nullptr, nullptr);
+    });
     grid_arrive(a, ++epoch);
-    prefetch_gemm(lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, C, 4 * C, nullptr, nullptr);
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += h Wfcproj + b
-    gemm_phase<false, false, false, KG1, 4 * KG1, JG>(a, lds, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs,
-                                                      a.h, nullptr, nullptr, a.x, a.x);
+    gemm_phase<false, false, false>(a, lds, w_fcproj, a.h, a.x, a.x, [&]() {
+      if (l + 1 < a.L)
+        load_phase_weights(w_qkv, a.qkvw + (l + 1) * 3 * cs * cs, a.qkvb + (l + 1) * 3 * cs,
+                           a.ln1w + (l + 1) * cs, a.ln1b + (l + 1) * cs);
+    });
     grid_arrive(a, ++epoch);
-    if (l + 1 < a.L)
-      prefetch_gemm(lds, a.qkvw + (l + 1) * 3 * cs * cs, a.qkvb + (l + 1) * 3 * cs, 3 * C, C,
-                    a.ln1w + (l + 1) * cs, a.ln1b + (l + 1) * cs);
-    else
-      prefetch_lm_head<ULM>(a, lds);
     if (!grid_wait(a, lds, epoch)) return;
   }
   lm_head_phase<4 * KG1, ULM>(a, lds);
@@ -751,9 +719,9 @@ int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) 
   const size_t lds = decode_step_lds_bytes(c, step.B, step.pos);
   const int jg = (step.B + 3) / 4, kg1 = c.channels / 256;
   const void* kernel = kg1 == 1   ? kernel_for<1, 8>(jg)
-                       : kg1 == 2 ? kernel_for<2, 16>(jg)
-                       : kg1 == 3 ? kernel_for<3, 24>(jg)
-                                  : kernel_for<4, 32>(jg);
+                       : kg1 == 2 ? kernel_for<2, 8>(jg)
+                       : kg1 == 3 ? kernel_for<3, 12>(jg)
+                                  : kernel_for<4, 16>(jg);
   static bool lds_raised[4][4] = {};
   if (lds > 48 * 1024 && !lds_raised[kg1 - 1][jg - 1]) {
     G2_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
