@@ -3,26 +3,22 @@
 //
 // Why one kernel.  A decode step streams every weight once (498 MB for GPT-2 124M: 62 us
 // at HBM speed) through 62 dependent matrix-vector-shaped operations.  As separate launches
-// each of them costs 7-12 us however little it does (dispatch, ramp, drain), 0.73 ms per
+// each of them costs 6-12 us however little it does (dispatch, ramp, drain), 0.61 ms per
 // step.  Inside one kernel the hand-over between two operations is a barrier across the
-// workgroups (~1.5 us, see below), and the next operation's weights are already on their
-// way into the L2 while the barrier is waited for.
+// workgroups (~2 us, see below), and the next operation's weights are already on their
+// way into registers while the current one computes.
 //
-// Work split.  Every workgroup (one per compute unit, 4 waves: one per SIMD) takes N / gridDim.x
-// consecutive weight rows (= output columns) of each GEMM for the whole K, at most 16 of
-// them: one 16x16 MFMA tile per workgroup whose K range is split over the 4 waves
-// (v_mfma_f32_16x16x4_f32, A = 16 weight rows, B = the <= 16 activation rows; partial
-// tiles summed through LDS in wave order, so results are deterministic).  No output is
-// shared between workgroups and nothing is reduced through memory.  The layernorms run
-// inside the GEMMs that consume them (every workgroup recomputes the statistics of the
-// <= 16 rows from the activations it loads anyway: llm.c's two passes, mean then
-// variance), the residual adds inside the GEMMs that produce the update, GELU in the fc
-// epilogue:
+// Work split.  The grid is exactly 256 workgroups of 4 waves (one wave per SIMD), one per
+// compute unit, all resident at once.  Every workgroup takes N / 256 consecutive weight rows
+// (= output columns) of each GEMM for the whole K: no output is shared between workgroups
+// and nothing is reduced through memory.  The layernorms run inside the GEMMs that consume
+// them (every workgroup recomputes the statistics of the <= 16 rows from the activations it
+// loads anyway: llm.c's two passes, mean then variance), the residual adds inside the GEMMs
+// that produce the update, GELU in the fc epilogue:
 //   qkv = LN1(x) Wqkv | attention over the cache | x += y Wproj | h = gelu(LN2(x) Wfc) |
 //   x += h Wfcproj
 // (Four waves, not sixteen: a phase is a few hundred instructions of bookkeeping per wave
-// around a few dozen loads and MFMAs, every wave repeats the bookkeeping, and with sixteen
-// waves that repetition -- not memory -- set the pace: 5.4 us per layernorm+GEMM phase.)
+// around a few dozen loads and MFMAs, and every wave repeats the bookkeeping.)
 // Attention takes one workgroup per (sequence, head): it appends the new key and value to
 // the cache and runs the softmax over positions 0..pos, 16 lanes per cache row.
 // The lm-head gives every wave 16-row groups of wte for the whole K (no cross-wave sum),
@@ -34,11 +30,11 @@
 // whole L2) made a grid barrier cost 12 us on this chip; instead the few KB of activations
 // are written and read with cache-bypassing accesses (sc0 sc1) and the barrier is an array
 // of per-workgroup epoch flags accessed the same way: a workgroup waits for its own
-// stores to be acknowledged, publishes the phase number, and polls everybody's flag
-// (1.5 us for 256 workgroups).  Weights and the cache rows of earlier steps are read-only
-// for the kernel and go through the caches normally.  Every wait is bounded: a
-// workgroup that spins too long raises an error word that makes every workgroup leave the
-// kernel, and the host reports it on the next call.
+// stores to be acknowledged, publishes the phase number, and polls everybody's flag.
+// Weights and the cache rows of earlier steps are read-only for the kernel and go through
+// the caches normally.  Every wait is bounded: a workgroup that spins too long raises an
+// error word that makes every workgroup leave the kernel, and the host reports it on a
+// later call.
 #include "common.hpp"
 
 namespace g2 {
