@@ -134,13 +134,16 @@ int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, 
 int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C);
 
 // One decode step as a single persistent kernel (decode.hip): every pointer is device memory.
+constexpr int kDecodeMaxBatch = 16;  // sequences the persistent decode-step kernel takes
 struct DecodeStep {
   const float *wte, *wpe_row, *ln1w, *ln1b, *qkvw, *qkvb, *attprojw, *attprojb, *ln2w, *ln2b, *fcw,
       *fcb, *fcprojw, *fcprojb, *lnfw, *lnfb;
   const int* ids;      // (B) new token of every sequence
   float* kv;           // keys of layer l at kv + 2*l*plane, values at kv + (2*l+1)*plane: (B, maxT, C)
   size_t plane;
-  float *x, *qkv, *atty, *h;  // (B,C) (B,3C) (B,C) (B,4C), handed between workgroups
+  // handed between workgroups: qkv (B,3C) row-major; x, atty (16,C) and h (16,4C) in granules
+  // of 4 sequences x 4 channels (see decode.hip)
+  float *x, *qkv, *atty, *h;
   float* logits;              // (B,V)
   unsigned* flags;            // [gridDim.x * FLAG_STRIDE] epochs, then the error word
   unsigned epoch0;            // flags hold values below epoch0 + 1 when the kernel starts

@@ -65,6 +65,7 @@ struct GPT2 {
   // its last launch ended with, a pinned host copy of the error word (refreshed after every
   // step, looked at on the next call)
   unsigned* step_flags;
+  float* step_act;  // its activations: x, attention output, hidden row, 16 sequences tall each
   unsigned step_epoch;
   unsigned* step_error_host;
   bool step_persistent;      // use the persistent kernel where it takes the model
@@ -107,6 +108,8 @@ static void free_cache(GPT2* m) {
   if (m->kv) (void)hipFree(m->kv);
   if (m->step_logits) (void)hipFree(m->step_logits);
   if (m->step_flags) (void)hipFree(m->step_flags);
+  if (m->step_act) (void)hipFree(m->step_act);
+  m->step_act = nullptr;
   if (m->step_error_host) (void)hipHostFree(m->step_error_host);
   m->kv = m->step_logits = nullptr;
   m->step_flags = m->step_error_host = nullptr;
@@ -125,6 +128,10 @@ static int reserve_cache(GPT2* m, int B) {
   const size_t flag_bytes = decode_step_flag_bytes(m->device);
   if (e == hipSuccess && flag_bytes) e = hipMalloc((void**)&m->step_flags, flag_bytes);
   if (e == hipSuccess && flag_bytes) e = hipMemset(m->step_flags, 0, flag_bytes);
+  // rows of sequences that do not exist are read (and ignored) by the kernel: keep them finite
+  const size_t act_bytes = (size_t)kDecodeMaxBatch * 6 * c.channels * sizeof(float);
+  if (e == hipSuccess) e = hipMalloc((void**)&m->step_act, act_bytes);
+  if (e == hipSuccess) e = hipMemset(m->step_act, 0, act_bytes);
   if (e == hipSuccess) e = hipHostMalloc((void**)&m->step_error_host, sizeof(unsigned), hipHostMallocDefault);
   if (e == hipSuccess) *m->step_error_host = 0;
   if (e != hipSuccess) {
@@ -557,7 +564,7 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
   float* other = m->res_b;
   G2_HIP(hipMemcpyAsync(m->ids, next_ids_device, (size_t)B * sizeof(int), hipMemcpyDeviceToDevice,
                         stream()));
-  const bool persistent = m->step_persistent && m->step_flags && decode_step_supported(c, B, m->device);
+  const bool persistent = m->step_persistent && m->step_flags && m->step_act && decode_step_supported(c, B, m->device);
   if (!persistent)  // the persistent kernel gathers the embeddings itself
     G2_TRY(encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
   const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
@@ -593,10 +600,10 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
     st.ids = m->ids;
     st.kv = m->kv;
     st.plane = plane;
-    st.x = residual;
+    st.x = m->step_act;
     st.qkv = m->qkv;
-    st.atty = m->atty;
-    st.h = m->fch;
+    st.atty = m->step_act + (size_t)kDecodeMaxBatch * cs;
+    st.h = m->step_act + (size_t)kDecodeMaxBatch * 2 * cs;
     st.logits = m->step_logits;
     st.flags = m->step_flags;
     st.epoch0 = m->step_epoch;
