@@ -46,9 +46,9 @@ constexpr int DS_GRID = 256;  // workgroups: the shapes below are compiled for e
 constexpr int FLAG_STRIDE = 16;  // one 64-byte line per workgroup's flag
 
 // LDS carve-up, in floats
-constexpr int LDS_STAT = 0;                               // [2][waves][16 rows]
-constexpr int LDS_SMALL = LDS_STAT + 2 * DS_WAVES * 16;   // [2][waves]: attention max / sum per wave
-constexpr int LDS_BAD = LDS_SMALL + 2 * DS_WAVES;         // one int: a wait timed out
+constexpr int LDS_STAT = 0;                               // [2][16 sequences][4 waves x 4 lane rows]
+constexpr int LDS_SMALL = LDS_STAT + 2 * 16 * 16;         // attention: max per (wave, lane row) [16] | sum per wave [4]
+constexpr int LDS_BAD = LDS_SMALL + 32;                   // one int: a wait timed out
 // GEMM phases: partial tiles [waves][NQ][64] | gamma, beta [2C]; attention: scores | partial
 // outputs; lm-head: normalised rows | gamma, beta
 constexpr int LDS_FREE = LDS_BAD + 32;
@@ -287,26 +287,27 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
   wait_vm();
   load_next();
   if (LN) {
-    // statistics of sequence 4*jg + r4: its row is spread over the 16 blocks of all 4 waves
+    // Statistics of sequence 4*jg + r4: its row is spread over the 16 blocks of all 4 waves.
+    // Two rotations inside each row of 16 lanes sum the row's 4 blocks; the 16 partial sums
+    // (4 waves x 4 lane rows) of a sequence meet in LDS.
     float* const stat = lds + LDS_STAT;
+    const int srow = wave * 4 + (lane >> 4);
     float mean[JG], rstd[JG];
 #pragma unroll
     for (int jg = 0; jg < JG; jg++) {
       float sum = 0.f;
 #pragma unroll
       for (int c = 0; c < KG; c++) sum += (xv[c][jg][0] + xv[c][jg][1]) + (xv[c][jg][2] + xv[c][jg][3]);
-      sum += __shfl_xor(sum, 4, 64);
-      sum += __shfl_xor(sum, 8, 64);
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
-      if (blk == 0) stat[wave * 16 + 4 * jg + r4] = sum;
+      sum += dpp<0x124>(sum);  // row_ror:4
+      sum += dpp<0x128>(sum);  // row_ror:8
+      if ((lane & 12) == 0) stat[(4 * jg + r4) * 16 + srow] = sum;
     }
     lds_barrier();  // not __syncthreads(): that would wait for the next phase's weights in flight
 #pragma unroll
     for (int jg = 0; jg < JG; jg++) {
-      float m = 0.f;
-#pragma unroll
-      for (int w = 0; w < DS_WAVES; w++) m += stat[w * 16 + 4 * jg + r4];
+      const f32x4* const p = reinterpret_cast<const f32x4*>(stat + (4 * jg + r4) * 16);
+      const f32x4 s4 = (p[0] + p[1]) + (p[2] + p[3]);
+      const float m = (s4[0] + s4[1]) + (s4[2] + s4[3]);
       mean[jg] = m / (float)K;
       float q = 0.f;
 #pragma unroll
@@ -314,18 +315,16 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
         const f32x4 d = xv[c][jg] - mean[jg];
         q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
       }
-      q += __shfl_xor(q, 4, 64);
-      q += __shfl_xor(q, 8, 64);
-      q += __shfl_xor(q, 16, 64);
-      q += __shfl_xor(q, 32, 64);
-      if (blk == 0) stat[DS_WAVES * 16 + wave * 16 + 4 * jg + r4] = q;
+      q += dpp<0x124>(q);
+      q += dpp<0x128>(q);
+      if ((lane & 12) == 0) stat[256 + (4 * jg + r4) * 16 + srow] = q;
     }
     lds_barrier();  // not __syncthreads(): that would wait for the next phase's weights in flight
 #pragma unroll
     for (int jg = 0; jg < JG; jg++) {
-      float var = 0.f;
-#pragma unroll
-      for (int w = 0; w < DS_WAVES; w++) var += stat[DS_WAVES * 16 + w * 16 + 4 * jg + r4];
+      const f32x4* const p = reinterpret_cast<const f32x4*>(stat + 256 + (4 * jg + r4) * 16);
+      const f32x4 s4 = (p[0] + p[1]) + (p[2] + p[3]);
+      const float var = (s4[0] + s4[1]) + (s4[2] + s4[3]);
       rstd[jg] = 1.0f / sqrtf(var / (float)K + 1e-5f);
     }
 #pragma unroll
@@ -373,9 +372,9 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
     }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      sum[j] += __shfl_xor(sum[j], 1, 64);
-      sum[j] += __shfl_xor(sum[j], 2, 64);
-      sum[j] += __shfl_xor(sum[j], 4, 64);
+      sum[j] += dpp<0xB1>(sum[j]);   // quad_perm [1,0,3,2]
+      sum[j] += dpp<0x4E>(sum[j]);   // quad_perm [2,3,0,1]
+      sum[j] += dpp<0x141>(sum[j]);  // row_half_mirror: the other quad of the 8 lanes
     }
     const int row = 4 * (q / (4 * JG)) + (q & 3), j0 = 4 * ((q >> 2) % JG);
     if (esub == 0 && q < NQ && row < ROWS) {
@@ -437,13 +436,18 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
       }
     }
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  if (lane == 0) small[wave] = mx;
+  // the 16 lanes of a row hold the same maximum; the 16 rows of the workgroup meet in LDS
+  if (sub == 0) small[wave * 4 + p4] = mx;
   __syncthreads();
-  float m = small[0];
-#pragma unroll
-  for (int w = 1; w < DS_WAVES; w++) m = fmaxf(m, small[w]);  // finite: position 0 always exists
+  float m;
+  {
+    const f32x4* const p = reinterpret_cast<const f32x4*>(small);
+    const f32x4 m4 = {fmaxf(fmaxf(p[0][0], p[1][0]), fmaxf(p[2][0], p[3][0])),
+                      fmaxf(fmaxf(p[0][1], p[1][1]), fmaxf(p[2][1], p[3][1])),
+                      fmaxf(fmaxf(p[0][2], p[1][2]), fmaxf(p[2][2], p[3][2])),
+                      fmaxf(fmaxf(p[0][3], p[1][3]), fmaxf(p[2][3], p[3][3]))};
+    m = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));  // finite: position 0 always exists
+  }
 
   float sum = 0.f;
   for (int t = tid; t <= pos; t += DS_THREADS) {
@@ -452,11 +456,11 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
     sum += e;
   }
   sum = wave_sum(sum);
-  if (lane == 0) small[DS_WAVES + wave] = sum;
+  if (lane == 0) small[16 + wave] = sum;
   __syncthreads();
   float l = 0.f;
 #pragma unroll
-  for (int w = 0; w < DS_WAVES; w++) l += small[DS_WAVES + w];
+  for (int w = 0; w < DS_WAVES; w++) l += small[16 + w];
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int g0 = wave; 4 * g0 <= pos; g0 += UN * DS_WAVES) {
@@ -471,17 +475,12 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
 #pragma unroll
     for (int u = 0; u < UN; u++) acc += pw[u] * vf[u];
   }
-#pragma unroll
-  for (int e = 0; e < 4; e++) {
-    acc[e] += __shfl_xor(acc[e], 16, 64);
-    acc[e] += __shfl_xor(acc[e], 32, 64);
-  }
-  if (p4 == 0) *reinterpret_cast<f32x4*>(part + wave * 64 + 4 * sub) = acc;
+  *reinterpret_cast<f32x4*>(part + tid * 4) = acc;  // [wave][lane row][64 channels]
   __syncthreads();
   if (tid < 64) {
     float o = 0.f;
 #pragma unroll
-    for (int w = 0; w < DS_WAVES; w++) o += part[w * 64 + tid];
+    for (int w = 0; w < 4 * DS_WAVES; w++) o += part[w * 64 + tid];
     store_bypass(a.atty + granule_index(b, head * 64 + tid, C), o / l);
   }
   __syncthreads();  // LDS is reused by the workgroup's next item
@@ -699,7 +698,7 @@ size_t decode_step_probe_slots(int num_layers) {
 static size_t decode_step_lds_bytes(const GPT2Config& c, int B, int pos) {
   const size_t C = c.channels, jg = (B + 3) / 4;
   const size_t gemm = 2 * C + DS_WAVES * ((C / 256) * jg * 4) * kWave;  // gamma, beta | partial tiles
-  const size_t att = (size_t)((pos + 64) & ~63) + DS_WAVES * 64;        // scores | partial outputs
+  const size_t att = (size_t)((pos + 64) & ~63) + 4 * DS_WAVES * 64;    // scores | partial outputs
   const size_t lm = (size_t)B * (C + 4) + 2 * C;                        // rows | gamma, beta
   size_t most = gemm > att ? gemm : att;
   if (lm > most) most = lm;
