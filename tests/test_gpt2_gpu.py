@@ -287,6 +287,9 @@ def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
     (dict(max_seq_len=300, vocab_size=1031, num_layers=3, num_heads=8, channels=512), 16, 250, 5),
     (dict(max_seq_len=64, vocab_size=50257, num_layers=2, num_heads=12, channels=768), 1, 1, 4),
     (dict(g2.GPT2_124M), 8, 120, 10),
+    # the cache attention's sweeps of 256 positions: steps across the first and second boundary
+    (dict(max_seq_len=600, vocab_size=211, num_layers=2, num_heads=4, channels=256), 2, 252, 8),
+    (dict(max_seq_len=600, vocab_size=211, num_layers=2, num_heads=4, channels=256), 3, 508, 8),
 ])
 def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_path(cfg, B, T0, steps):
     print(f"persistent decode cfg={cfg} B={B} T0={T0} steps={steps}", flush=True)
