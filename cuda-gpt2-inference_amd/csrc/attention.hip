@@ -389,8 +389,9 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(float* out, cons
 }
 
 // ---- one new position per sequence against a key/value cache ---------------------
-// Keys and values of past positions live in kc / vc, (B, maxT, C) each, written by
-// kv_store_kernel (a whole prompt) and by this kernel (the new position).  One workgroup
+// Keys and values of past positions live in kc / vc, (B, NH, maxT, hs) each -- the rows of one
+// (sequence, head) are consecutive in memory, so that a step streams them as one block --
+// written by kv_store_kernel (a whole prompt) and by this kernel (the new position).  One workgroup
 // of 16 waves per (sequence, head): it appends the new key and value, computes the pos+1
 // scores one wave per position (lanes over the head dimension, DPP reduction), turns them
 // into softmax weights in LDS, and accumulates the weighted values with each wave taking
@@ -411,12 +412,12 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode_kernel(
   float* const sc = dec_lds;
   float* const part = dec_lds + ((pos + 64) & ~63);
   const float* qrow = qkv + (size_t)b * 3 * C + head * hs;
-  float* const kb = kc + (size_t)b * maxT * C + head * hs;
-  float* const vb = vc + (size_t)b * maxT * C + head * hs;
+  float* const kb = kc + (size_t)blockIdx.x * maxT * hs;
+  float* const vb = vc + (size_t)blockIdx.x * maxT * hs;
 
   for (int d = tid; d < hs; d += DEC_WAVES * kWave) {
-    kb[(size_t)pos * C + d] = qrow[C + d];
-    vb[(size_t)pos * C + d] = qrow[2 * C + d];
+    kb[(size_t)pos * hs + d] = qrow[C + d];
+    vb[(size_t)pos * hs + d] = qrow[2 * C + d];
   }
   float qv[4];
 #pragma unroll
@@ -430,7 +431,7 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode_kernel(
 #pragma unroll
     for (int u = 0; u < 4; u++) {
       const int t = min(t0 + u * DEC_WAVES, pos);
-      const float* kr = kb + (size_t)t * C;
+      const float* kr = kb + (size_t)t * hs;
       p[u] = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; j++)
@@ -474,7 +475,7 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode_kernel(
     for (int u = 0; u < 4; u++) {
       const int t = t0 + u * DEC_WAVES;
       pw[u] = (t <= pos) ? sc[t] : 0.f;
-      const float* vr = vb + (size_t)min(t, pos) * C;
+      const float* vr = vb + (size_t)min(t, pos) * hs;
 #pragma unroll
       for (int j = 0; j < 4; j++) vv[u][j] = (lane + 64 * j < hs) ? vr[lane + 64 * j] : 0.f;
     }
@@ -514,12 +515,12 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
   float* const sc = dec_lds;
   float* const part = dec_lds + ((pos + 64) & ~63);
   const float* qrow = qkv + (size_t)b * 3 * C + head * 64;
-  float* const kb = kc + (size_t)b * maxT * C + head * 64 + 4 * sub;
-  float* const vb = vc + (size_t)b * maxT * C + head * 64 + 4 * sub;
+  float* const kb = kc + (size_t)blockIdx.x * maxT * 64 + 4 * sub;
+  float* const vb = vc + (size_t)blockIdx.x * maxT * 64 + 4 * sub;
 
   if (tid < 16) {
-    *reinterpret_cast<f32x4*>(kb + (size_t)pos * C) = *reinterpret_cast<const f32x4*>(qrow + C + 4 * sub);
-    *reinterpret_cast<f32x4*>(vb + (size_t)pos * C) =
+    *reinterpret_cast<f32x4*>(kb + (size_t)pos * 64) = *reinterpret_cast<const f32x4*>(qrow + C + 4 * sub);
+    *reinterpret_cast<f32x4*>(vb + (size_t)pos * 64) =
         *reinterpret_cast<const f32x4*>(qrow + 2 * C + 4 * sub);
   }
   const f32x4 q4 = *reinterpret_cast<const f32x4*>(qrow + 4 * sub);
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
       const int t = min(4 * (g0 + u * DEC_WAVES) + p4, pos);
-      kf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb + (size_t)t * C));
+      kf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb + (size_t)t * 64));
     }
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
@@ -573,7 +574,7 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
     for (int u = 0; u < DEC_UNROLL; u++) {
       const int t = 4 * (g0 + u * DEC_WAVES) + p4;
       pw[u] = (t <= pos) ? sc[t] : 0.f;
-      vf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb + (size_t)min(t, pos) * C));
+      vf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb + (size_t)min(t, pos) * 64));
     }
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) acc += pw[u] * vf[u];
@@ -594,17 +595,18 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
 }
 
 // Copies the key and value thirds of a prompt's packed qkv (B, T, 3C) into the cache
-// (B, maxT, C each) at positions 0..T-1.
+// (B, NH, maxT, hs each) at positions 0..T-1.
 __global__ __launch_bounds__(256) void kv_store_kernel(float* __restrict__ kc, float* __restrict__ vc,
                                                         const float* __restrict__ qkv, int T,
-                                                        int maxT, int C, size_t total) {
+                                                        int maxT, int C, int hs, size_t total) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
   const size_t bt = i / C;
   const int c = (int)(i - bt * C);
   const size_t b = bt / T, t = bt - b * T;
   const float* src = qkv + bt * 3 * C + C + c;
-  const size_t dst = (b * maxT + t) * C + c;
+  const int head = c / hs, d = c - head * hs;
+  const size_t dst = ((b * (size_t)(C / hs) + head) * maxT + t) * hs + d;
   kc[dst] = src[0];
   vc[dst] = src[C];
 }
@@ -630,11 +632,12 @@ int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, 
   return GPT2HIP_OK;
 }
 
-int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C) {
+int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C, int NH) {
   const size_t total = (size_t)B * T * C;
   if (total == 0) return GPT2HIP_OK;
+  if (NH < 1 || C % NH != 0) return fail(GPT2HIP_EINVAL, "kv_store: bad shape C=%d NH=%d", C, NH);
   hipLaunchKernelGGL(kv_store_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream(), kc,
-                     vc, qkv, T, maxT, C, total);
+                     vc, qkv, T, maxT, C, C / NH, total);
   G2_LAUNCH_CHECK("kv_store");
   return GPT2HIP_OK;
 }

@@ -127,23 +127,28 @@ int skinny_launch(float* out, const float* inp, const float* weight, const float
                   bool gelu);
 
 // Decode-step attention of one new position per sequence against the key/value cache
-// (kc, vc: (B, maxT, C)); appends the new key/value at `pos`.  qkv is (B, 3C).
+// (kc, vc: (B, NH, maxT, hs)); appends the new key/value at `pos`.  qkv is (B, 3C).
 int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, int B, int pos,
                             int maxT, int C, int NH);
 // Copies a prompt's keys and values from packed qkv (B, T, 3C) into the cache.
-int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C);
+int kv_store_launch(float* kc, float* vc, const float* qkv, int B, int T, int maxT, int C, int NH);
 
 // One decode step as a single persistent kernel (decode.hip): every pointer is device memory.
 constexpr int kDecodeMaxBatch = 16;  // sequences the persistent decode-step kernel takes
+constexpr int kDecodeMaxSplits = 4;  // ranges of positions per (sequence, head) in its attention phase
 struct DecodeStep {
   const float *wte, *wpe_row, *ln1w, *ln1b, *qkvw, *qkvb, *attprojw, *attprojb, *ln2w, *ln2b, *fcw,
       *fcb, *fcprojw, *fcprojb, *lnfw, *lnfb;
   const int* ids;      // (B) new token of every sequence
-  float* kv;           // keys of layer l at kv + 2*l*plane, values at kv + (2*l+1)*plane: (B, maxT, C)
+  float* kv;           // keys of layer l at kv + 2*l*plane, values at kv + (2*l+1)*plane: (B, NH, maxT, 64)
   size_t plane;
   // handed between workgroups: qkv (B,3C) row-major; x, atty (16,C) and h (16,4C) in granules
   // of 4 sequences x 4 channels (see decode.hip)
   float *x, *qkv, *atty, *h;
+  // attention in att_splits > 1 ranges per (sequence, head): their unnormalised outputs
+  // (att_splits x the layout of atty) and (maximum, sum) pairs
+  float *att_part, *att_ml;
+  int att_splits;
   float* logits;              // (B,V)
   unsigned* flags;            // [gridDim.x * FLAG_STRIDE] epochs, then the error word
   unsigned epoch0;            // flags hold values below epoch0 + 1 when the kernel starts
@@ -159,6 +164,8 @@ struct DecodeStep {
 // uses barrier epochs step.epoch0 + 1 .. step.epoch0 + 5 * L.
 bool decode_step_supported(const GPT2Config& c, int B, int device);
 size_t decode_step_flag_bytes(int device);
+size_t decode_step_activation_floats(const GPT2Config& c);      // DecodeStep::x .. att_ml, one buffer
+int decode_step_attention_splits(const GPT2Config& c, int B, int pos);  // DecodeStep::att_splits
 size_t decode_step_probe_slots(int num_layers);  // clock slots DecodeStep::trace needs
 int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device);
 

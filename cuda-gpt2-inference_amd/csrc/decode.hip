@@ -90,6 +90,10 @@ __device__ __forceinline__ void store_bypass(float* p, float v) {
 __device__ __forceinline__ int granule_index(int seq, int channel, int channels) {
   return (seq >> 2) * 4 * channels + (channel >> 2) * 16 + (seq & 3) * 4 + (channel & 3);
 }
+// (maximum, sum) of range `split` of (sequence, head): the four sequences of a group side by side
+__device__ __forceinline__ int split_stat_index(int split, int seq, int head, int heads) {
+  return (((split * (kDecodeMaxBatch / 4) + (seq >> 2)) * heads + head) * 4 + (seq & 3)) * 2;
+}
 // Workgroup barrier that orders LDS traffic only (no wait for global loads in flight).
 __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
@@ -201,6 +205,51 @@ __device__ __forceinline__ void load_phase_weights(PhaseWeights<ROWS, KG, JG, LN
   }
 }
 
+// The input of the projection phase when attention ran in S ranges per (sequence, head): the
+// ranges' results combined, x = sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m).
+// K = C, and a wave's group c of 64 k is exactly head wave * KG + c.  All loads are issued
+// before anything is combined.
+template <int S, int KG, int JG>
+__device__ __forceinline__ void merge_splits(const DecodeStep& a, f32x4 (&xv)[KG][JG], int wave, int lane) {
+  const int K = a.C, r4 = lane & 3;
+  const Bypass part(a.att_part, (size_t)S * kDecodeMaxBatch * K);
+  const int xoff = wave * (KG * 256) + 4 * lane;
+  unsigned long long ml[JG][KG][S];
+  f32x4 os[JG][KG][S];
+#pragma unroll
+  for (int jg = 0; jg < JG; jg++)
+#pragma unroll
+    for (int c = 0; c < KG; c++)
+#pragma unroll
+      for (int sp = 0; sp < S; sp++) {
+        const float* p = a.att_ml + split_stat_index(sp, 4 * jg + r4, wave * KG + c, a.NH);
+        ml[jg][c][sp] = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+        os[jg][c][sp] = part.load4(sp * kDecodeMaxBatch * K + jg * 4 * K + xoff + c * 256);
+      }
+#pragma unroll
+  for (int jg = 0; jg < JG; jg++)
+#pragma unroll
+    for (int c = 0; c < KG; c++) {
+      float ms[S], ls[S], mmax = -INFINITY;
+#pragma unroll
+      for (int sp = 0; sp < S; sp++) {
+        ms[sp] = __builtin_bit_cast(float, (unsigned)(ml[jg][c][sp] & 0xffffffffu));
+        ls[sp] = __builtin_bit_cast(float, (unsigned)(ml[jg][c][sp] >> 32));
+        mmax = fmaxf(mmax, ms[sp]);
+      }
+      f32x4 num = {0.f, 0.f, 0.f, 0.f};
+      float den = 0.f;
+#pragma unroll
+      for (int sp = 0; sp < S; sp++) {
+        const float e = expf(ms[sp] - mmax);
+        num += e * os[jg][c][sp];
+        den += e * ls[sp];
+      }
+      xv[c][jg] = num / den;  // sequences past B: whatever the buffers hold, never stored
+    }
+}
+
 // out[j][n0 + i] = resid + act( LN(in)[j] . W[n0 + i] + bias ) for this workgroup's ROWS output
 // columns n0 = ROWS * blockIdx.x, on v_mfma_f32_4x4x1_16B_f32: sixteen independent 4x4 outer
 // products per instruction, block b of lanes 4b..4b+3.  Lane (b, r) feeds weight row 4*rg + r
@@ -217,7 +266,10 @@ __device__ __forceinline__ void load_phase_weights(PhaseWeights<ROWS, KG, JG, LN
 // GATHER: the input rows are wte[ids[j]] + wpe[pos] (the first phase of a step); workgroup 0
 // also stores them as the residual stream x.  `in` and `resid` are in the granule layout, and
 // so is `out` unless ROWMAJOR_OUT (qkv, which attention reads a head at a time).
-template <bool LN, bool GELU, bool GATHER, bool ROWMAJOR_OUT, int ROWS, int KG, int JG, typename LoadNext>
+// MERGE: the projection phase; with a.att_splits > 1 its input is combined from attention's
+// ranges (merge_splits) instead of loaded from `in`.
+template <bool LN, bool GELU, bool GATHER, bool ROWMAJOR_OUT, bool MERGE, int ROWS, int KG, int JG,
+          typename LoadNext>
 __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
                                            const PhaseWeights<ROWS, KG, JG, LN>& pw, const float* in, float* out,
                                            const float* resid, LoadNext&& load_next) {
@@ -233,21 +285,16 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
   float* const gb = red + DS_WAVES * NQ * kWave;  // gamma [K] | beta [K], with LN only
 
   // Epilogue role: threads 8q..8q+7 sum register q (+32 per pass) over blocks and waves; the
-  // first of them finishes the four outputs (row 4*rg + v, sequences 4*jg .. 4*jg+3).
+  // first four of them finish one output each (row 4*rg + v, sequence 4*jg + esub).
   const int eq = tid >> 3, esub = tid & 7;
-  float rs[NIT][4];
+  float rs[NIT];
+  bool mine[NIT];
 #pragma unroll
   for (int it = 0; it < NIT; it++) {
-    const int q = eq + 32 * it, row = 4 * (q / (4 * JG)) + (q & 3), j0 = 4 * ((q >> 2) % JG);
-#pragma unroll
-    for (int j = 0; j < 4; j++) rs[it][j] = 0.f;
-    if (esub == 0 && q < NQ && row < ROWS) {
-      if (resid != nullptr) {
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-          if (j0 + j < B) rs[it][j] = load_bypass(resid + granule_index(j0 + j, n0 + row, N));
-      }
-    }
+    const int q = eq + 32 * it, row = 4 * (q / (4 * JG)) + (q & 3), j = 4 * ((q >> 2) % JG) + esub;
+    mine[it] = esub < 4 && q < NQ && row < ROWS && j < B;
+    rs[it] = 0.f;
+    if (resid != nullptr && mine[it]) rs[it] = load_bypass(resid + granule_index(j, n0 + row, N));
   }
 
   // this lane's first float of the wave's quarter of K
@@ -257,8 +304,21 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
   f32x4 xv[KG][JG];
   const Bypass xin(GATHER ? a.x : in, (size_t)4 * JG * K);
   const int xoff = wave * (KG * 256) + 4 * lane;
+  // (the combinations the host asks for: up to 4 ranges with at most 4 sequences, 2 with at
+  // most 8, none beyond: every combination is code that all phases share the instruction
+  // cache with)
+  const bool merge = MERGE && JG <= 2 && a.att_splits > 1;
+  if (merge) {
+    if (JG > 1 || a.att_splits == 2)
+      merge_splits<2, KG, JG>(a, xv, wave, lane);
+    else if (a.att_splits == 3)
+      merge_splits<3, KG, JG>(a, xv, wave, lane);
+    else
+      merge_splits<4, KG, JG>(a, xv, wave, lane);
+  }
 #pragma unroll
   for (int jg = 0; jg < JG; jg++) {
+    if (merge) break;
     if (GATHER) {
       const int bj = min(4 * jg + r4, B - 1);
       const int id = a.ids[bj];
@@ -376,61 +436,69 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
       sum[j] += dpp<0x4E>(sum[j]);   // quad_perm [2,3,0,1]
       sum[j] += dpp<0x141>(sum[j]);  // row_half_mirror: the other quad of the 8 lanes
     }
-    const int row = 4 * (q / (4 * JG)) + (q & 3), j0 = 4 * ((q >> 2) % JG);
-    if (esub == 0 && q < NQ && row < ROWS) {
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (j0 + j < B) {
-          float val = sum[j] + pw.bias[it];
-          if (GELU) val = gelu_tanh(val);
-          store_bypass(out + (ROWMAJOR_OUT ? (j0 + j) * N + n0 + row : granule_index(j0 + j, n0 + row, N)),
-                       val + rs[it][j]);
-        }
+    const int row = 4 * (q / (4 * JG)) + (q & 3), j = 4 * ((q >> 2) % JG) + esub;
+    if (mine[it]) {
+      float val = (esub == 0 ? sum[0] : esub == 1 ? sum[1] : esub == 2 ? sum[2] : sum[3]) + pw.bias[it];
+      if (GELU) val = gelu_tanh(val);
+      store_bypass(out + (ROWMAJOR_OUT ? j * N + n0 + row : granule_index(j, n0 + row, N)), val + rs[it]);
     }
   }
 }
 
-// One (sequence, head) of attention against the cache, head size 64: appends the new key and
-// value (taken from the qkv row other workgroups just wrote), scores positions 0..pos with
-// 16 lanes per cache row (a wave instruction covers four positions, 16 of them in flight),
-// softmax through LDS, weighted values the same way.
+// Attention of one new position against the cache, head size 64.  A compute unit streams
+// cache rows at ~35 GB/s however many loads it keeps in flight, so at long contexts B * NH
+// workgroups alone would leave the phase waiting for a third of the chip: from
+// kSplitFromPos positions on, a (sequence, head) is cut into S = a.att_splits consecutive
+// ranges of positions, one workgroup each.  Every range runs its own softmax -- maximum m,
+// sum l, unnormalised weighted values o -- and stores (m, l, o); the projection phase
+// combines the ranges when it loads its input (merge_splits).  With S = 1 the normalised
+// result is stored as that phase's input directly.
+//
+// One range [tb, te]: 16 lanes hold one cache row, a wave instruction covers four positions,
+// 16 of them in flight; scores go through LDS, weighted values the same way.  The range that
+// ends at the new position appends the new key and value (taken from the qkv row other
+// workgroups just wrote) to the cache first.
 __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, float* kc, float* vc,
-                                               int b, int head) {
+                                               int b, int head, int split) {
   constexpr int UN = 16;
   const int tid = opaque_tid(), lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int p4 = lane >> 4, sub = lane & 15;
-  const int C = a.C, pos = a.pos;
+  const int C = a.C, pos = a.pos, S = a.att_splits;
+  // ranges are multiples of four positions long; S > 1 only where every range is non-empty
+  const int chunk = S == 1 ? pos + 1 : (((pos + S) / S + 3) & ~3);
+  const int tb = split * chunk, te = min(pos, tb + chunk - 1), n = te - tb + 1;
   float* const sc = lds + LDS_FREE;
-  float* const part = sc + ((pos + 64) & ~63);
+  float* const part = sc + ((n + 63) & ~63);
   float* const small = lds + LDS_SMALL;
   const float scale = 0.125f;
-  float* const kb = kc + (size_t)b * a.maxT * C + head * 64 + 4 * sub;
-  float* const vb = vc + (size_t)b * a.maxT * C + head * 64 + 4 * sub;
+  // the cache is (B, NH, maxT, 64): the rows of this (sequence, head) are consecutive
+  float* const kb = kc + ((size_t)(b * a.NH + head) * a.maxT + tb) * 64 + 4 * sub;
+  float* const vb = vc + ((size_t)(b * a.NH + head) * a.maxT + tb) * 64 + 4 * sub;
 
   const Bypass qkv(a.qkv, (size_t)a.B * 3 * C);
   const int qi = b * 3 * C + head * 64 + 4 * sub;
   const f32x4 q4 = qkv.load4(qi);
-  if (tid < 16) {
-    *reinterpret_cast<f32x4*>(kb + (size_t)pos * C) = qkv.load4(qi + C);
-    *reinterpret_cast<f32x4*>(vb + (size_t)pos * C) = qkv.load4(qi + 2 * C);
+  if (te == pos && tid < 16) {
+    *reinterpret_cast<f32x4*>(kb + (size_t)(n - 1) * 64) = qkv.load4(qi + C);
+    *reinterpret_cast<f32x4*>(vb + (size_t)(n - 1) * 64) = qkv.load4(qi + 2 * C);
   }
   __syncthreads();  // the appended row is visible to the whole workgroup
 
   float mx = -INFINITY;
-  for (int g0 = wave; 4 * g0 <= pos; g0 += UN * DS_WAVES) {
+  for (int g0 = wave; 4 * g0 < n; g0 += UN * DS_WAVES) {
     f32x4 kf[UN];
 #pragma unroll
     for (int u = 0; u < UN; u++) {
-      const int t = min(4 * (g0 + u * DS_WAVES) + p4, pos);
-      kf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb + (size_t)t * C));
+      const int t = min(4 * (g0 + u * DS_WAVES) + p4, n - 1);
+      kf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb + (size_t)t * 64));
     }
 #pragma unroll
     for (int u = 0; u < UN; u++) {
       const int t = 4 * (g0 + u * DS_WAVES) + p4;
       const f32x4 pr = q4 * kf[u];
       const float sv = row16_sum((pr[0] + pr[1]) + (pr[2] + pr[3])) * scale;
-      if (t <= pos) {
+      if (t < n) {
         if (sub == 0) sc[t] = sv;
         mx = fmaxf(mx, sv);
       }
@@ -446,11 +514,11 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
                       fmaxf(fmaxf(p[0][1], p[1][1]), fmaxf(p[2][1], p[3][1])),
                       fmaxf(fmaxf(p[0][2], p[1][2]), fmaxf(p[2][2], p[3][2])),
                       fmaxf(fmaxf(p[0][3], p[1][3]), fmaxf(p[2][3], p[3][3]))};
-    m = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));  // finite: position 0 always exists
+    m = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));  // finite: the range is not empty
   }
 
   float sum = 0.f;
-  for (int t = tid; t <= pos; t += DS_THREADS) {
+  for (int t = tid; t < n; t += DS_THREADS) {
     const float e = expf(sc[t] - m);
     sc[t] = e;
     sum += e;
@@ -463,14 +531,14 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
   for (int w = 0; w < DS_WAVES; w++) l += small[16 + w];
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int g0 = wave; 4 * g0 <= pos; g0 += UN * DS_WAVES) {
+  for (int g0 = wave; 4 * g0 < n; g0 += UN * DS_WAVES) {
     f32x4 vf[UN];
     float pw[UN];
 #pragma unroll
     for (int u = 0; u < UN; u++) {
       const int t = 4 * (g0 + u * DS_WAVES) + p4;
-      pw[u] = (t <= pos) ? sc[t] : 0.f;
-      vf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb + (size_t)min(t, pos) * C));
+      pw[u] = (t < n) ? sc[t] : 0.f;
+      vf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb + (size_t)min(t, n - 1) * 64));
     }
 #pragma unroll
     for (int u = 0; u < UN; u++) acc += pw[u] * vf[u];
@@ -481,9 +549,13 @@ __device__ __forceinline__ void attention_item(const DecodeStep& a, float* lds, 
     float o = 0.f;
 #pragma unroll
     for (int w = 0; w < 4 * DS_WAVES; w++) o += part[w * 64 + tid];
-    store_bypass(a.atty + granule_index(b, head * 64 + tid, C), o / l);
+    if (S == 1) {
+      store_bypass(a.atty + granule_index(b, head * 64 + tid, C), o / l);
+    } else {
+      store_bypass(a.att_part + (size_t)split * kDecodeMaxBatch * C + granule_index(b, head * 64 + tid, C), o);
+      if (tid < 2) store_bypass(a.att_ml + split_stat_index(split, b, head, a.NH) + tid, tid == 0 ? m : l);
+    }
   }
-  __syncthreads();  // LDS is reused by the workgroup's next item
 }
 
 // logits = LNf(x) . wte^T.  The normalised rows go to LDS once per workgroup; wave w then
@@ -621,7 +693,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
   if (*reinterpret_cast<int*>(lds + LDS_BAD) != 0) return;
   unsigned epoch = a.epoch0;
 
-  const int items = a.B * a.NH;  // (sequence, head) pairs of the attention phase
+  const int items = a.B * a.NH * a.att_splits;  // (sequence, head, range) triples of the attention phase
   PhaseWeights<3 * KG1, KG1, JG, true> w_qkv;
   PhaseWeights<KG1, KG1, JG, false> w_proj;
   PhaseWeights<4 * KG1, KG1, JG, true> w_fc;
@@ -634,34 +706,38 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
     // qkv = LN1(x) Wqkv + b
     auto next_proj = [&]() { load_phase_weights(w_proj, a.attprojw + l * cs * cs, a.attprojb + l * cs, nullptr, nullptr); };
     if (l == 0)
-      gemm_phase<true, false, true, true>(a, lds, w_qkv, nullptr, a.qkv, nullptr, next_proj);
+      gemm_phase<true, false, true, true, false>(a, lds, w_qkv, nullptr, a.qkv, nullptr, next_proj);
     else
-      gemm_phase<true, false, false, true>(a, lds, w_qkv, a.x, a.qkv, nullptr, next_proj);
+      gemm_phase<true, false, false, true, false>(a, lds, w_qkv, a.x, a.qkv, nullptr, next_proj);
     grid_arrive(a, ++epoch);
     if (!grid_wait(a, lds, epoch)) return;
 
     // attention over the cache
-    for (int item = blockIdx.x; item < items; item += gridDim.x)
-      attention_item(a, lds, kc, vc, item / a.NH, item % a.NH);
+    // at most one item per workgroup: B <= 16 sequences of at most 1024 / 64 heads, and the
+    // host splits only as far as the grid goes
+    if ((int)blockIdx.x < items) {
+      const int bh = (int)blockIdx.x / a.att_splits;
+      attention_item(a, lds, kc, vc, bh / a.NH, bh % a.NH, (int)blockIdx.x % a.att_splits);
+    }
     grid_arrive(a, ++epoch);
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += y Wproj + b
-    gemm_phase<false, false, false, false>(a, lds, w_proj, a.atty, a.x, a.x, [&]() {
+    gemm_phase<false, false, false, false, true>(a, lds, w_proj, a.atty, a.x, a.x, [&]() {
       load_phase_weights(w_fc, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, a.ln2w + l * cs, a.ln2b + l * cs);
     });
     grid_arrive(a, ++epoch);
     if (!grid_wait(a, lds, epoch)) return;
 
     // h = gelu(LN2(x) Wfc + b)
-    gemm_phase<true, true, false, false>(a, lds, w_fc, a.x, a.h, nullptr, [&]() {
+    gemm_phase<true, true, false, false, false>(a, lds, w_fc, a.x, a.h, nullptr, [&]() {
       load_phase_weights(w_fcproj, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, nullptr, nullptr);
     });
     grid_arrive(a, ++epoch);
     if (!grid_wait(a, lds, epoch)) return;
 
     // x += h Wfcproj + b
-    gemm_phase<false, false, false, false>(a, lds, w_fcproj, a.h, a.x, a.x, [&]() {
+    gemm_phase<false, false, false, false, false>(a, lds, w_fcproj, a.h, a.x, a.x, [&]() {
       if (l + 1 < a.L)
         load_phase_weights(w_qkv, a.qkvw + (l + 1) * 3 * cs * cs, a.qkvb + (l + 1) * 3 * cs,
                            a.ln1w + (l + 1) * cs, a.ln1b + (l + 1) * cs);
@@ -693,6 +769,26 @@ size_t decode_step_flag_bytes(int device) {
 
 size_t decode_step_probe_slots(int num_layers) {
   return (size_t)DS_GRID * TRACE_SLOTS * (5 * (size_t)num_layers + 1);
+}
+
+// Ranges per (sequence, head) of the attention phase at position pos.  Splitting pays from a
+// few hundred positions on (the projection phase loads S results instead of one: +1.8 us).
+constexpr int kSplitFromPos = 384;
+int decode_step_attention_splits(const GPT2Config& c, int B, int pos) {
+  if (pos < kSplitFromPos) return 1;
+  const int s = DS_GRID / (B * c.num_heads);  // as far as the grid goes
+  if (s < 2 || B > 8) return 1;  // the kernel combines ranges only for up to 8 sequences,
+  if (B > 4) return 2;           // and more than 2 of them only for up to 4
+  return s > kDecodeMaxSplits ? kDecodeMaxSplits : s;
+}
+
+// Floats of the activation buffer the kernel hands data between workgroups in: x, attention
+// output, hidden row (granule layout, 16 sequences tall), the attention ranges' partial
+// outputs and their (maximum, sum) pairs.
+size_t decode_step_activation_floats(const GPT2Config& c) {
+  const size_t C = c.channels;
+  return (size_t)kDecodeMaxBatch * (6 + kDecodeMaxSplits) * C +
+         (size_t)kDecodeMaxSplits * kDecodeMaxBatch * c.num_heads * 2;
 }
 
 static size_t decode_step_lds_bytes(const GPT2Config& c, int B, int pos) {

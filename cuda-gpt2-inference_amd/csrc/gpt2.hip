@@ -54,7 +54,7 @@ struct GPT2 {
   int last_B, last_T;
   bool last_has_logits;
 
-  // key/value cache of the incremental (prefill + decode) path: (L, 2, kv_batch, maxT, C),
+  // key/value cache of the incremental (prefill + decode) path: (L, 2, kv_batch, NH, maxT, hs),
   // and the logits of the newest position, (kv_batch, V)
   float* kv;
   float* step_logits;
@@ -65,7 +65,7 @@ struct GPT2 {
   // its last launch ended with, a pinned host copy of the error word (refreshed after every
   // step, looked at on the next call)
   unsigned* step_flags;
-  float* step_act;  // its activations: x, attention output, hidden row, 16 sequences tall each
+  float* step_act;  // the activations it hands between workgroups (decode_step_activation_floats)
   unsigned step_epoch;
   unsigned* step_error_host;
   bool step_persistent;      // use the persistent kernel where it takes the model
@@ -129,7 +129,7 @@ static int reserve_cache(GPT2* m, int B) {
   if (e == hipSuccess && flag_bytes) e = hipMalloc((void**)&m->step_flags, flag_bytes);
   if (e == hipSuccess && flag_bytes) e = hipMemset(m->step_flags, 0, flag_bytes);
   // rows of sequences that do not exist are read (and ignored) by the kernel: keep them finite
-  const size_t act_bytes = (size_t)kDecodeMaxBatch * 6 * c.channels * sizeof(float);
+  const size_t act_bytes = decode_step_activation_floats(c) * sizeof(float);
   if (e == hipSuccess) e = hipMalloc((void**)&m->step_act, act_bytes);
   if (e == hipSuccess) e = hipMemset(m->step_act, 0, act_bytes);
   if (e == hipSuccess) e = hipHostMalloc((void**)&m->step_error_host, sizeof(unsigned), hipHostMallocDefault);
@@ -230,7 +230,7 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
     if (fill_cache) {
       const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
       G2_TRY(kv_store_launch(m->kv + (2 * (size_t)l) * plane, m->kv + (2 * (size_t)l + 1) * plane, m->qkv,
-                             B, T, c.max_seq_len, C));
+                             B, T, c.max_seq_len, C, NH));
     }
     G2_STEP(GPT2_PROF_ATTENTION, attention_forward_status(m->atty, nullptr, nullptr, m->qkv, B, T, C, NH));
     G2_STEP(GPT2_PROF_MATMUL_ATTPROJ, matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs,
@@ -604,6 +604,9 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
     st.qkv = m->qkv;
     st.atty = m->step_act + (size_t)kDecodeMaxBatch * cs;
     st.h = m->step_act + (size_t)kDecodeMaxBatch * 2 * cs;
+    st.att_part = m->step_act + (size_t)kDecodeMaxBatch * 6 * cs;
+    st.att_ml = st.att_part + (size_t)kDecodeMaxBatch * kDecodeMaxSplits * cs;
+    st.att_splits = decode_step_attention_splits(c, B, pos);
     st.logits = m->step_logits;
     st.flags = m->step_flags;
     st.epoch0 = m->step_epoch;

@@ -290,6 +290,11 @@ def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
     # the cache attention's sweeps of 256 positions: steps across the first and second boundary
     (dict(max_seq_len=600, vocab_size=211, num_layers=2, num_heads=4, channels=256), 2, 252, 8),
     (dict(max_seq_len=600, vocab_size=211, num_layers=2, num_heads=4, channels=256), 3, 508, 8),
+    # long contexts cut every (sequence, head) into ranges of positions: 4, 3 and 2 of them
+    (dict(max_seq_len=400, vocab_size=211, num_layers=2, num_heads=4, channels=256), 1, 380, 8),
+    (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=16, channels=1024), 3, 390, 3),
+    (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=8, channels=512), 7, 391, 3),
+    (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=8, channels=512), 13, 391, 3),
 ])
 def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_path(cfg, B, T0, steps):
     print(f"persistent decode cfg={cfg} B={B} T0={T0} steps={steps}", flush=True)
