@@ -19,8 +19,9 @@
 //   x += h Wfcproj
 // (Four waves, not sixteen: a phase is a few hundred instructions of bookkeeping per wave
 // around a few dozen loads and MFMAs, and every wave repeats the bookkeeping.)
-// Attention takes one workgroup per (sequence, head): it appends the new key and value to
-// the cache and runs the softmax over positions 0..pos, 16 lanes per cache row.
+// Attention takes one workgroup per (sequence, head) -- at long contexts one per range of
+// positions of a (sequence, head) -- which appends the new key and value to the cache and
+// runs the softmax over its positions, 16 lanes per cache row.
 // The lm-head gives every wave 16-row groups of wte for the whole K (no cross-wave sum),
 // with the normalised activations staged in LDS.
 //
