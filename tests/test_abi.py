@@ -69,3 +69,12 @@ def test_synthetic_params_match_oracle_layout():
     assert list(sizes) == list(syn.PARAM_NAMES)
     for k in sizes:
         assert sizes[k] == int(np.prod(shapes[k]))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits (before touching a GPU)."""
+    import subprocess, sys
+    bench = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")
+    proc = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode != 0
+    assert "--gpus 1" in (proc.stdout + proc.stderr)
