@@ -16,10 +16,14 @@ constexpr int kWavesPerBlock = 4;  // 256 threads
 // NV float4 per lane cover C <= 256*NV.  FUSED adds inp2 and stores the sum.  A wave
 // owns ROWS consecutive rows and issues all of their loads before it touches any of
 // them: at N = 8192 four rows per wave (a quarter of the waves, four times the bytes
-// in flight per wave) moved 72-76 % of HBM peak against 62-67 % for one row per wave.
+// in flight per wave) moved 71 % of HBM peak against 62-67 % for one row per wave, and at
+// C = 1024 eight rows per wave 75 % against 70.6 % for four (at C = 768 eight change
+// nothing).  The plain form, with half the traffic per row, does best with two rows per
+// wave and streaming (non-temporal) stores: 68 / 72 % at C = 768 / 1024 against 65 / 63 %.
 // EXACT (C == 256*NV and N % ROWS == 0, true for GPT-2) removes every bounds check, so
 // that the loads are issued as one unconditional batch.
-template <int NV, int ROWS, bool FUSED, bool EXACT>
+// NTS: non-temporal stores.
+template <int NV, int ROWS, bool FUSED, bool EXACT, bool NTS>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
     float* res_out, float* out, float* __restrict__ mean, float* __restrict__ rstd,
     const float* inp1, const float* inp2, const float* __restrict__ weight,
@@ -60,7 +64,12 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
 #pragma unroll
       for (int j = 0; j < NV; j++) {
         const int c = lane + j * kWave;
-        if (EXACT || c < C4) ro[c] = v[r][j];
+        if (EXACT || c < C4) {
+          if (NTS)
+            __builtin_nontemporal_store(v[r][j], ro + c);
+          else
+            ro[c] = v[r][j];
+        }
       }
     }
 
@@ -92,7 +101,10 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
       const int c = lane + j * kWave;
       if (EXACT || c < C4) {
         const f32x4 n = (v[r][j] - m) * rs;
-        o[c] = n * w4[c] + b4[c];
+        if (NTS)
+          __builtin_nontemporal_store(n * w4[c] + b4[c], o + c);
+        else
+          o[c] = n * w4[c] + b4[c];
       }
     }
   }
@@ -152,19 +164,25 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   const bool vec = (C % 4 == 0) && C <= 4096 && aligned16(out) && aligned16(inp1) &&
                    aligned16(weight) && aligned16(bias) &&
                    (!FUSED || (aligned16(res_out) && aligned16(inp2)));
-  // four rows per wave once there are enough rows to still fill the chip
+  // several rows per wave once there are enough rows to still fill the chip
   const bool wide = N >= 4096;
-#define G2_LN(NV, ROWS, EXACT)                                                                  \
-  hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED, EXACT>),                           \
+#define G2_LN(NV, ROWS, EXACT, NTS)                                                             \
+  hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED, EXACT, NTS>),                      \
                      dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, stream(), \
                      res_out, out, mean, rstd, inp1, inp2, weight, bias, N, C)
-#define G2_LN_ROWS(NV)                         \
-  if (wide && C == 256 * NV && N % 4 == 0) {   \
-    G2_LN(NV, 4, true);                        \
-  } else if (wide) {                           \
-    G2_LN(NV, 4, false);                       \
-  } else {                                     \
-    G2_LN(NV, 1, false);                       \
+#define G2_LN_ROWS(NV)                                              \
+  if (wide && C == 256 * NV && N % 8 == 0) {                        \
+    if (!FUSED) {                                                   \
+      G2_LN(NV, 2, true, true);                                     \
+    } else if (NV == 4) {                                           \
+      G2_LN(NV, 8, true, false);                                    \
+    } else {                                                        \
+      G2_LN(NV, 4, true, false);                                    \
+    }                                                               \
+  } else if (wide) {                                                \
+    G2_LN(NV, 4, false, false);                                     \
+  } else {                                                          \
+    G2_LN(NV, 1, false, false);                                     \
   }
   if (!vec) {
     hipLaunchKernelGGL((layernorm_rows_generic_kernel<FUSED>),
@@ -181,7 +199,7 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   } else if (C <= 2048) {
     G2_LN_ROWS(8)
   } else {
-    G2_LN(16, 1, false);
+    G2_LN(16, 1, false, false);
   }
 #undef G2_LN_ROWS
 #undef G2_LN
