@@ -86,17 +86,23 @@ def forward_bytes(cfg, B, T):
 LAUNCHES = {"encoder": 1, "layernorm": 1, "matmul_lmhead": 1}
 
 
-def time_launch(g2, fn, iters=30, warmup=10):
-    """Median-free simple average: HIP events on the null stream around `iters` launches."""
+def time_launch(g2, fn, iters=30, warmup=10, groups=5):
+    """HIP events on the null stream around `iters` back-to-back launches, `groups` times; the
+    median group's average per launch (one group in five catches a clock or host hiccup)."""
     import torch
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    t = g2.Timer()
-    t.start()
-    for i in range(iters):
-        fn(warmup + i)
-    return t.stop_ms() / iters
+    per_launch = []
+    n = warmup
+    for _ in range(groups):
+        t = g2.Timer()
+        t.start()
+        for i in range(iters):
+            fn(n + i)
+        per_launch.append(t.stop_ms() / iters)
+        n += iters
+    return sorted(per_launch)[len(per_launch) // 2]
 
 
 def standalone(g2):
