@@ -66,26 +66,16 @@ __device__ __forceinline__ float dpp(float v) {
       float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 
-// Lane CTRL-selected value of `v` for the rows in ROW_MASK, 0 for the other rows.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_rows(float v) {
-  return __builtin_bit_cast(
-      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
-}
-
-// All-lanes sum over a 64-wide wavefront, without a trip through the LDS pipeline: four
-// DPP steps inside each row of 16 lanes (quad swaps, half-row mirror, row mirror), then
-// row 1 and row 3 add their left neighbour's total (row_bcast:15), rows 2 and 3 the total of
-// the lower half (row_bcast:31); lane 63 then holds (r0 + r1) + (r2 + r3) -- the pairing of
-// an xor-16, xor-32 butterfly -- and is broadcast through a scalar register.
+// All-lanes sum over a 64-wide wavefront: four DPP steps inside each row of 16
+// lanes (quad swaps, half-row mirror, row mirror), then two cross-row exchanges.
 __device__ __forceinline__ float wave_sum(float v) {
   v += dpp<0xB1>(v);   // quad_perm [1,0,3,2]
   v += dpp<0x4E>(v);   // quad_perm [2,3,0,1]
   v += dpp<0x141>(v);  // row_half_mirror
   v += dpp<0x140>(v);  // row_mirror
-  v += dpp_rows<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-  v += dpp_rows<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
 }
 
 // Sum over each row of 16 lanes (all 16 lanes of the row receive it).
@@ -111,14 +101,9 @@ __device__ __forceinline__ float wave_max(float v) {
   v = fmaxf(v, dpp<0x4E>(v));
   v = fmaxf(v, dpp<0x141>(v));
   v = fmaxf(v, dpp<0x140>(v));
-  // rows outside the mask keep their own value (old = v)
-  const int b15 = __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xa,
-                                              0xf, false);
-  v = fmaxf(v, __builtin_bit_cast(float, b15));
-  const int b31 = __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xc,
-                                              0xf, false);
-  v = fmaxf(v, __builtin_bit_cast(float, b31));
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  v = fmaxf(v, __shfl_xor(v, 32, 64));
+  return v;
 }
 
 // tanh-GELU, 0.5x(1+tanh(u)) with u = sqrt(2/pi)(x + 0.044715x^3), the formula of

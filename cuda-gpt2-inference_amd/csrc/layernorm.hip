@@ -54,6 +54,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
 
   const f32x4* w4 = reinterpret_cast<const f32x4*>(weight);
   const f32x4* b4 = reinterpret_cast<const f32x4*>(bias);
+  float my_mean = 0.f, my_rstd = 0.f;  // lane r keeps the statistics of the wave's row r
 #pragma unroll
   for (int r = 0; r < ROWS; r++) {
     const int row = row0 + r;
@@ -90,7 +91,12 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
     const float var = wave_sum(q) / (float)C;
     const float rs = 1.0f / sqrtf(var + 1e-5f);
 
-    if (lane == 0) {
+    if (FUSED) {
+      if (lane == r) {
+        my_mean = m;
+        my_rstd = rs;
+      }
+    } else if (lane == 0) {
       if (mean) mean[row] = m;
       if (rstd) rstd[row] = rs;
     }
@@ -107,6 +113,13 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
           o[c] = n * w4[c] + b4[c];
       }
     }
+  }
+  // fused form: one store of ROWS consecutive floats per wave and array instead of one per
+  // row (77 % of HBM peak against 75-76 % at C = 1024; the plain form, with two rows per
+  // wave, was slower with it)
+  if (FUSED && lane < ROWS && (EXACT || row0 + lane < N)) {
+    if (mean) mean[row0 + lane] = my_mean;
+    if (rstd) rstd[row0 + lane] = my_rstd;
   }
 }
 
