@@ -203,15 +203,16 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device);
 /* How gpt2_decode runs (no counterpart in the reference).  persistent != 0 (the default): one
  * persistent kernel per step where it takes the model (up to 16 sequences, head size 64,
  * channels 256, 512, 768 or 1024, a device with at least 256 compute units), otherwise one
- * launch per operation; 0: always one launch per operation.  spin_limit bounds the polls a workgroup of the persistent kernel
- * spends on one flag of its grid barrier before it gives up and ends the kernel (default
- * 2^21); a step that gave up makes the NEXT gpt2_decode call fail and empties the cache. */
+ * launch per operation; 0: always one launch per operation.  spin_limit bounds the polls a
+ * workgroup of the persistent kernel spends on one flag of its grid barrier before it gives
+ * up and ends the kernel (default 2^21); a step that gave up makes the NEXT gpt2_decode call
+ * fail and empties the cache. */
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit);
 /* One gpt2_decode step of the persistent kernel with a clock probe: every workgroup g records
  * the 100 MHz wall clock when it has finished the work of phase p (clocks[(2p) * G + g]) and
  * when it has passed the grid barrier after it (clocks[(2p + 1) * G + g]); phases are, per
  * layer, qkv GEMM, attention, projection GEMM, fc GEMM, fc projection GEMM, then the lm-head
- * (work only).  G = compute units of the device; gpt2_decode_probe_size() = the slots needed
+ * (work only).  G = 256, the kernel's workgroups; gpt2_decode_probe_size() = the slots needed
  * (0 if the persistent kernel does not take the model at the prefilled batch size). */
 int gpt2_decode_probe_status(GPT2* model, const int* next_ids_device, unsigned long long* clocks_device,
                              size_t capacity);
