@@ -826,8 +826,8 @@ int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) 
   const size_t lds = decode_step_lds_bytes(c, step.B, step.pos);
   const int jg = (step.B + 3) / 4, kg1 = c.channels / 256;
   const void* kernel = kg1 == 1   ? kernel_for<1, 8>(jg)
-                       : kg1 == 2 ? kernel_for<2, 8>(jg)
-                       : kg1 == 3 ? kernel_for<3, 12>(jg)
+                       : kg1 == 2 ? kernel_for<2, 16>(jg)
+                       : kg1 == 3 ? kernel_for<3, 24>(jg)
                                   : kernel_for<4, 16>(jg);
   static bool lds_raised[4][4] = {};
   if (lds > 48 * 1024 && !lds_raised[kg1 - 1][jg - 1]) {
