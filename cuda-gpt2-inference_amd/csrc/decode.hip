@@ -575,6 +575,16 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   const int K = a.C, B = a.B, V = a.V;
   const int ldx = K + 4;  // row stride of the staged activations
   float* const xs = lds + LDS_FREE;
+  // Every group is NCH (even) chunks of UC units.  One chunk is always in flight ahead of the
+  // MFMAs, across group boundaries too: while the last chunk of a group is multiplied, the
+  // first chunk of the wave's next group is already loading -- and the very first chunk loads
+  // while the layernorm below runs (its barriers do not wait for loads in flight).
+  constexpr int NCH = 4 * U1 / UC;
+  static_assert(NCH * UC == 4 * U1 && NCH % 2 == 0, "a group is an even number of chunks");
+  const int step = (int)gridDim.x * DS_WAVES;
+  int cg = lm_head_first_group(wave);
+  f32x4 wa[UC], wb[UC];
+  const float* wp = a.wte + (size_t)min(cg * 16 + r16, V - 1) * K + 4 * kq;
   {
     const size_t koff = (size_t)wave * (U1 * 16) + 4 * kq;
     float* const gb = xs + (size_t)B * ldx;  // gamma [K] | beta [K], shared by all rows
@@ -589,6 +599,11 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
 #pragma unroll
       for (int c = 0; c < U1; c++) xv[c] = xin.load4(xi + c * 64);
     }
+    if (cg * 16 < V) {
+#pragma unroll
+      for (int c = 0; c < UC; c++)
+        wa[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)c * 16));
+    }
     float* const stat = lds + LDS_STAT;
     float sum = 0.f;
 #pragma unroll
@@ -596,7 +611,7 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     if (kq == 0) stat[wave * 16 + r16] = sum;
-    __syncthreads();
+    lds_barrier();
     float mean = 0.f;
 #pragma unroll
     for (int w = 0; w < DS_WAVES; w++) mean += stat[w * 16 + r16];
@@ -610,7 +625,7 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
     q += __shfl_xor(q, 16, 64);
     q += __shfl_xor(q, 32, 64);
     if (kq == 0) stat[DS_WAVES * 16 + wave * 16 + r16] = q;
-    __syncthreads();
+    lds_barrier();
     float var = 0.f;
 #pragma unroll
     for (int w = 0; w < DS_WAVES; w++) var += stat[DS_WAVES * 16 + w * 16 + r16];
@@ -622,24 +637,10 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
             (xv[c] - mean) * rstd * *reinterpret_cast<const f32x4*>(gb + koff + c * 16) +
             *reinterpret_cast<const f32x4*>(gb + K + koff + c * 16);
     }
-    __syncthreads();
+    lds_barrier();
   }
 
-  // Every group is NCH (even) chunks of UC units.  One chunk is always in flight ahead of the
-  // MFMAs, across group boundaries too: while the last chunk of a group is multiplied, the
-  // first chunk of the wave's next group is already loading.
-  constexpr int NCH = 4 * U1 / UC;
-  static_assert(NCH * UC == 4 * U1 && NCH % 2 == 0, "a group is an even number of chunks");
   const float* const xrow = xs + (size_t)min(r16, B - 1) * ldx + 4 * kq;
-  const int step = (int)gridDim.x * DS_WAVES;
-  int cg = lm_head_first_group(wave);
-  f32x4 wa[UC], wb[UC];
-  const float* wp = a.wte + (size_t)min(cg * 16 + r16, V - 1) * K + 4 * kq;
-  if (cg * 16 < V) {
-#pragma unroll
-    for (int c = 0; c < UC; c++)
-      wa[c] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + (size_t)c * 16));
-  }
   for (; cg * 16 < V; cg += step) {
     const int n0 = cg * 16;
     const float* const wnext = a.wte + (size_t)min(n0 + step * 16 + r16, V - 1) * K + 4 * kq;
