@@ -27,3 +27,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(scope="session", autouse=True)
+def _built_libraries():
+    """The tests load what is built; only when nothing is do they build it (in-tree, with
+    hipcc cross-compiling for gfx950: no GPU is needed for that)."""
+    import importlib
+    g2 = importlib.import_module("cuda-gpt2-inference_amd")
+    if not os.path.exists(g2.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    yield
