@@ -393,6 +393,9 @@ def main():
     import torch
     g2 = importlib.import_module("cuda-gpt2-inference_amd")
     syn = importlib.import_module("cuda-gpt2-inference_amd.synthetic")
+    if not os.path.exists(g2.LIB_PATH):  # load what is built; build only if nothing is
+        import __graft_entry__
+        __graft_entry__.build()
     if not torch.cuda.is_available():
         print("bench.py: no GPU", file=sys.stderr)
         sys.exit(2)
