@@ -244,6 +244,18 @@ def test_matmul_lm_head_no_bias():
     assert np.abs(got - ref).max() < 3e-5
 
 
+def test_matmul_scaling_the_input_by_two_scales_the_output_exactly():
+    """A property that holds at any size with no oracle: multiplying by a power of two is
+    exact in fp32, so out(2 x) must equal 2 out(x) bit for bit -- at the full lm-head size."""
+    M, C, OC = 8192, 768, 50257
+    say(f"matmul scaling property M={M} C={C} OC={OC}")
+    x, w, _ = mm_inputs(M, C, OC, 122, bias=False)
+    out1 = run_matmul(x, w, None)
+    out2 = run_matmul(2.0 * x, w, None)
+    assert torch.equal(out2, 2.0 * out1)
+    del out1, out2
+
+
 def test_matmul_generic_path_unaligned_k():
     x, w, b = mm_inputs(33, 30, 17, 122)  # C % 4 != 0
     assert_close(run_matmul(x, w, b), oracle.matmul_forward(x, w, b), "matmul generic")
@@ -330,6 +342,24 @@ def test_attention_other_head_sizes(B, T, NH, hs):
     out = torch.empty((B, T, C), device="cuda")
     g2.attention_forward(out, None, None, dev(qkv), B, T, C, NH)
     assert_close(out, oracle.attention_forward(qkv, NH), "attention generic")
+
+
+def test_attention_scaling_the_values_by_two_scales_the_output_exactly():
+    """Size-independent property at the benchmark shape: the output is linear in v, and
+    doubling is exact in fp32, so doubling v must double the output bit for bit."""
+    B, T, NH = 8, 1024, 12
+    C = NH * 64
+    say(f"attention scaling property B={B} T={T} NH={NH}")
+    qkv = np.random.default_rng(131).standard_normal((B, T, 3 * C), dtype=np.float32)
+    qkv2 = qkv.copy()
+    qkv2[:, :, 2 * C:] *= 2.0
+    outs = []
+    for a in (qkv, qkv2):
+        out = torch.empty(B, T, C, device="cuda")
+        g2.attention_forward(out, None, None, dev(a), B, T, C, NH)
+        outs.append(out)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[1], 2.0 * outs[0])
 
 
 def test_attention_large_scores_stay_finite():
