@@ -333,22 +333,25 @@ int gpt2_load_params_host(GPT2* model, const float* host_params, size_t n) {
 namespace g2 {
 
 // Reads and validates the 256-word header; on success *padded_v is the number of wte
-// rows stored in the file.
-static int read_checkpoint_header(FILE* f, const char* path, GPT2Config* cfg, int* padded_v) {
+// rows stored in the file and *elem_bytes the size of a stored parameter: 4 (fp32, versions
+// 1 and 3) or 2 (bf16, version 5, which widens to fp32 exactly).
+static int read_checkpoint_header(FILE* f, const char* path, GPT2Config* cfg, int* padded_v,
+                                  int* elem_bytes) {
   int header[256];
   if (fread(header, sizeof(int), 256, f) != 256)
     return fail(GPT2HIP_EINVAL, "checkpoint %s: shorter than its 1024-byte header", path);
   if (header[0] != 20240326)
     return fail(GPT2HIP_EINVAL, "checkpoint %s: bad magic %d (want 20240326)", path, header[0]);
-  if (header[1] != 1 && header[1] != 3)
-    return fail(GPT2HIP_EINVAL, "checkpoint %s: version %d is not an fp32 checkpoint (1 or 3)", path,
-                header[1]);
+  if (header[1] != 1 && header[1] != 3 && header[1] != 5)
+    return fail(GPT2HIP_EINVAL, "checkpoint %s: version %d is neither an fp32 (1, 3) nor a bf16 (5) checkpoint",
+                path, header[1]);
+  *elem_bytes = header[1] == 5 ? 2 : 4;
   cfg->max_seq_len = header[2];
   cfg->vocab_size = header[3];
   cfg->num_layers = header[4];
   cfg->num_heads = header[5];
   cfg->channels = header[6];
-  *padded_v = (header[1] == 3) ? header[7] : header[3];
+  *padded_v = (header[1] == 1) ? header[3] : header[7];
   if (cfg->max_seq_len < 1 || cfg->vocab_size < 1 || cfg->num_layers < 1 || cfg->num_heads < 1 ||
       cfg->channels < 1 || cfg->channels % cfg->num_heads != 0 || *padded_v < cfg->vocab_size)
     return fail(GPT2HIP_EINVAL, "checkpoint %s: implausible header (maxT %d V %d L %d NH %d C %d Vp %d)",
@@ -363,8 +366,8 @@ int gpt2_checkpoint_read_config(const char* path, GPT2Config* config) {
   if (!path || !config) return fail(GPT2HIP_EINVAL, "gpt2_checkpoint_read_config: null pointer");
   FILE* f = fopen(path, "rb");
   if (!f) return fail(GPT2HIP_EINVAL, "cannot open checkpoint %s", path);
-  int padded_v = 0;
-  const int rc = read_checkpoint_header(f, path, config, &padded_v);
+  int padded_v = 0, elem_bytes = 0;
+  const int rc = read_checkpoint_header(f, path, config, &padded_v, &elem_bytes);
   fclose(f);
   return rc;
 }
@@ -381,24 +384,35 @@ GPT2* gpt2_build_from_checkpoint(const char* path) {
     return nullptr;
   }
   GPT2Config cfg;
-  int padded_v = 0;
+  int padded_v = 0, elem_bytes = 0;
   GPT2* m = nullptr;
-  if (read_checkpoint_header(f, path, &cfg, &padded_v) == GPT2HIP_OK && (m = gpt2_create(&cfg))) {
+  if (read_checkpoint_header(f, path, &cfg, &padded_v, &elem_bytes) == GPT2HIP_OK && (m = gpt2_create(&cfg))) {
     // Stream the file through a bounded host buffer; skip wte's pad rows.
     const size_t C = cfg.channels;
     const size_t chunk = 16u << 20;  // floats
     std::vector<float> buf(chunk);
+    std::vector<unsigned short> half(elem_bytes == 2 ? chunk : 0);
     size_t done = 0;  // floats written to the device buffer
     bool ok = true;
     while (ok && done < m->num_params) {
       if (done == (size_t)cfg.vocab_size * C && padded_v > cfg.vocab_size)
-        ok = fseek(f, (long)((size_t)(padded_v - cfg.vocab_size) * C * sizeof(float)), SEEK_CUR) == 0;
+        ok = fseek(f, (long)((size_t)(padded_v - cfg.vocab_size) * C * (size_t)elem_bytes), SEEK_CUR) == 0;
       // never read across the end of wte, so that the pad can be skipped exactly there
       size_t want = std::min(chunk, m->num_params - done);
       if (done < (size_t)cfg.vocab_size * C) want = std::min(want, (size_t)cfg.vocab_size * C - done);
-      if (ok && fread(buf.data(), sizeof(float), want, f) != want) {
+      const size_t got = !ok ? 0
+                         : elem_bytes == 2 ? fread(half.data(), 2, want, f)
+                                           : fread(buf.data(), sizeof(float), want, f);
+      if (ok && got != want) {
         fail(GPT2HIP_EINVAL, "checkpoint %s: truncated (needs %zu parameters)", path, m->num_params);
         ok = false;
+      }
+      if (ok && elem_bytes == 2) {
+        // bf16 is the upper half of an fp32: widening is exact
+        for (size_t i = 0; i < want; i++) {
+          const unsigned bits = (unsigned)half[i] << 16;
+          memcpy(&buf[i], &bits, sizeof(float));
+        }
       }
       if (ok && hipMemcpy(m->params + done, buf.data(), want * sizeof(float),
                           hipMemcpyHostToDevice) != hipSuccess) {

@@ -62,19 +62,35 @@ def make_tokens(seed: int, B: int, T: int, vocab_size: int) -> np.ndarray:
 
 def write_llmc_checkpoint(path, flat_params: np.ndarray, *, version: int = 3, pad_to: int = 128,
                           pad_value: float = 7.5, **config) -> None:
-    """Write parameters as an llm.c checkpoint file: 256 int32 header words, then fp32
-    tensors.  Version 3 pads wte's rows to a multiple of pad_to (filled with pad_value,
-    which a correct loader must never let through); version 1 does not pad."""
+    """Write parameters as an llm.c checkpoint file: 256 int32 header words, then the
+    tensors.  Versions 3 (fp32) and 5 (bf16: the upper 16 bits of each fp32, so pass
+    parameters that are bf16-representable) pad wte's rows to a multiple of pad_to (filled
+    with pad_value, which a correct loader must never let through); version 1 (fp32) does
+    not pad."""
     V, C = config["vocab_size"], config["channels"]
-    Vp = -(-V // pad_to) * pad_to if version == 3 else V
+    Vp = -(-V // pad_to) * pad_to if version in (3, 5) else V
     header = np.zeros(256, np.int32)
     header[:7] = [20240326, version, config["max_seq_len"], V, config["num_layers"],
                   config["num_heads"], C]
-    if version == 3:
+    if version in (3, 5):
         header[7] = Vp
+
+    def stored(a):
+        a = np.ascontiguousarray(a, np.float32)
+        if version == 5:
+            return (a.view(np.uint32) >> 16).astype(np.uint16).tobytes()
+        return a.tobytes()
+
     with open(path, "wb") as f:
         f.write(header.tobytes())
-        f.write(np.ascontiguousarray(flat_params[:V * C], np.float32).tobytes())
+        f.write(stored(flat_params[:V * C]))
         if Vp > V:
-            f.write(np.full((Vp - V) * C, pad_value, np.float32).tobytes())
-        f.write(np.ascontiguousarray(flat_params[V * C:], np.float32).tobytes())
+            f.write(stored(np.full((Vp - V) * C, pad_value, np.float32)))
+        f.write(stored(flat_params[V * C:]))
+
+
+def round_to_bf16(a: np.ndarray) -> np.ndarray:
+    """fp32 values rounded to the nearest bf16 (ties to even), returned as fp32."""
+    bits = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return bits.astype(np.uint32).view(np.float32)

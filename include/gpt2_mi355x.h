@@ -159,11 +159,12 @@ float* gpt2_params_device(GPT2* model);
 /* Copies n = gpt2_num_parameters floats from host memory into that buffer. */
 int gpt2_load_params_host(GPT2* model, const float* host_params, size_t n);
 
-/* llm.c checkpoint files (gpt2_124M.bin): 256 int32 header words {20240326, version,
- * maxT, V, L, NH, C, padded V, ...} followed by the fp32 tensors in the order above.
- * Version 3 stores wte with its rows padded to "padded V" (the pad rows are skipped
- * on load: this library keeps wte unpadded); version 1 has no padding.  Other
- * versions (bf16) are rejected.  gpt2_checkpoint_read_config touches no GPU.
+/* llm.c checkpoint files (gpt2_124M.bin, gpt2_124M_bf16.bin): 256 int32 header words
+ * {20240326, version, maxT, V, L, NH, C, padded V, ...} followed by the tensors in the
+ * order above.  Version 3 (fp32) and version 5 (bf16, widened to fp32 on load, which is
+ * exact) store wte with its rows padded to "padded V" (the pad rows are skipped on load:
+ * this library keeps wte unpadded); version 1 (fp32) has no padding.  Other versions are
+ * rejected.  gpt2_checkpoint_read_config touches no GPU.
  * gpt2_build_from_checkpoint mirrors llm.c's function of that name
  * (gpt2_build_from_checkpoint(GPT2*, const char*)); it returns NULL on failure. */
 int gpt2_checkpoint_read_config(const char* path, GPT2Config* config);

@@ -15,14 +15,15 @@ syn = importlib.import_module("cuda-gpt2-inference_amd.synthetic")
 CFG = dict(max_seq_len=32, vocab_size=331, num_layers=2, num_heads=2, channels=128)
 
 
-@pytest.mark.parametrize("version", [1, 3])
+@pytest.mark.parametrize("version", [1, 3, 5])
 def test_header_roundtrip(tmp_path, version):
     params = syn.make_params(5, **CFG)
     path = tmp_path / f"v{version}.bin"
     syn.write_llmc_checkpoint(path, params, version=version, **CFG)
     assert g2.read_checkpoint_config(path) == CFG
-    pad_rows = (-CFG["vocab_size"]) % 128 if version == 3 else 0
-    assert path.stat().st_size == 1024 + 4 * (params.size + pad_rows * CFG["channels"])
+    pad_rows = (-CFG["vocab_size"]) % 128 if version != 1 else 0
+    elem = 2 if version == 5 else 4
+    assert path.stat().st_size == 1024 + elem * (params.size + pad_rows * CFG["channels"])
 
 
 def test_header_rejections(tmp_path):
@@ -40,8 +41,8 @@ def test_header_rejections(tmp_path):
 
     with pytest.raises(g2.GPT2HipError, match="bad magic"):
         g2.read_checkpoint_config(variant("magic.bin", 0, 1234))
-    with pytest.raises(g2.GPT2HipError, match="version 5"):
-        g2.read_checkpoint_config(variant("bf16.bin", 1, 5))
+    with pytest.raises(g2.GPT2HipError, match="version 4"):
+        g2.read_checkpoint_config(variant("v4.bin", 1, 4))
     with pytest.raises(g2.GPT2HipError, match="implausible"):
         g2.read_checkpoint_config(variant("heads.bin", 5, 3))      # C % NH != 0
     with pytest.raises(g2.GPT2HipError, match="implausible"):
@@ -55,10 +56,12 @@ def test_header_rejections(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("version", [1, 3])
+@pytest.mark.parametrize("version", [1, 3, 5])
 def test_checkpoint_model_equals_directly_loaded_model(tmp_path, version):
     import torch
     params = syn.make_params(6, perturb_affine=True, **CFG)
+    if version == 5:  # a bf16 file: its parameters widen to fp32 exactly
+        params = syn.round_to_bf16(params)
     path = tmp_path / "model.bin"
     syn.write_llmc_checkpoint(path, params, version=version, **CFG)
     ids = syn.make_tokens(7, 2, 32, CFG["vocab_size"])
