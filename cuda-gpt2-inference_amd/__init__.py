@@ -387,6 +387,21 @@ class GPT2:
         _check(lib().gpt2_decode_status(self._h, _i32(next_ids_device)), "gpt2_decode")
         return self.step_logits()
 
+    def generate_greedy(self, prompt_device, steps: int):
+        """Greedy continuation of a (B,T) prompt of device ids by `steps` tokens: prefill, then
+        argmax_forward over the step logits and one decode step per token, all queued on the
+        stream with no host synchronisation in between.  Returns (B, steps) int32 device ids."""
+        import torch
+        B, T = prompt_device.shape
+        V = self.config.vocab_size
+        out = torch.empty((steps, B), dtype=torch.int32, device="cuda")
+        logits = self.prefill(prompt_device)
+        for s in range(steps):
+            argmax_forward(out[s], logits, B, V)
+            if s + 1 < steps:
+                logits = self.decode(out[s])
+        return out.t().contiguous()
+
     def decode_probe(self, next_ids_device):
         """One decode step of the persistent kernel with its clock probe: returns a
         (phases, 2, workgroups) int64 tensor of 100 MHz wall-clock readings (work done / barrier

@@ -329,6 +329,30 @@ def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_
     finally:
         model.close()
 
+@pytest.mark.parametrize("persistent", [True, False])
+def test_gpt2_greedy_generation_equals_greedy_decoding_by_full_forward_passes(persistent):
+    """Prefill + argmax + decode steps, chained on the device, against the same continuation
+    produced the slow way: a full forward pass over the growing sequences for every token."""
+    cfg = dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=4, channels=256)
+    B, T0, steps = 3, 9, 12
+    print(f"greedy generation persistent={persistent}", flush=True)
+    params = syn.make_params(95, perturb_affine=True, **cfg)
+    prompt = torch.from_numpy(syn.make_tokens(96, B, T0, cfg["vocab_size"])).cuda()
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(params)
+        model.decode_options(persistent=persistent)
+        got = model.generate_greedy(prompt, steps)
+        seq = prompt.clone()
+        for s in range(steps):
+            nxt = model.forward_argmax(seq)[:, -1:].contiguous()
+            seq = torch.cat([seq, nxt], dim=1).contiguous()
+        want = seq[:, T0:]
+        assert torch.equal(got, want), (got.cpu(), want.cpu())
+    finally:
+        model.close()
+
+
 def test_gpt2_persistent_decode_gives_up_a_barrier_wait_cleanly():
     """Failure handling of the persistent kernel's grid barrier, forced from the host: with a
     spin limit of 0 the first workgroup that has to wait gives up, every workgroup leaves the
