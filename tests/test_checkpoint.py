@@ -1,8 +1,10 @@
 """llm.c checkpoint files: header parsing (CPU) and loading (GPU).
 
-The files are written here with numpy in llm.c's on-disk layout (256 int32 header
-words, fp32 tensors in checkpoint order, wte rows padded in version 3), independently
-of the loader under test.
+Most files are written by the package's own synthetic.write_llmc_checkpoint (256 int32
+header words, tensors in checkpoint order, wte rows padded in versions 3 and 5); the
+"literal layout" tests at the end build a file byte by byte from offsets written in this
+file, so that the loader is also checked against a layout it shares no code with.  No file
+produced by llm.c itself is available offline: agreement with one is not pinned.
 """
 import importlib
 
@@ -90,3 +92,83 @@ def test_truncated_checkpoint_is_an_error(tmp_path):
     path.write_bytes(data[:len(data) // 2])
     with pytest.raises(g2.GPT2HipError, match="truncated"):
         g2.GPT2.from_checkpoint(path)
+
+
+# ---------------------------------------------------------------------------------------
+# A file laid out from literal byte offsets, sharing nothing with synthetic.write_llmc_checkpoint
+# (so that the loader and the package's own writer cannot agree on a common mistake).
+# llm.c's train_gpt2.c documents the layout: a 1024-byte header of little-endian int32 words,
+# word 0 magic 20240326, 1 version, 2 max_seq_len, 3 vocab_size, 4 num_layers, 5 num_heads,
+# 6 channels, 7 padded_vocab_size; then the sixteen tensors, wte with padded_vocab_size rows.
+# No llm.c-produced file exists offline, so the format itself stays unpinned by upstream data.
+LIT = dict(max_seq_len=8, vocab_size=130, num_layers=2, num_heads=2, channels=64)
+LIT_VP = 256
+
+
+def _literal_tensors():
+    """(name, shape, values) in file order; tensor k holds k + 1 + (flat index mod 251) / 256,
+    all exactly representable in bf16-free fp32 and distinct between tensors."""
+    maxT, V, L, C = LIT["max_seq_len"], LIT["vocab_size"], LIT["num_layers"], LIT["channels"]
+    shapes = [("wte", (V, C)), ("wpe", (maxT, C)), ("ln1w", (L, C)), ("ln1b", (L, C)),
+              ("qkvw", (L, 3 * C, C)), ("qkvb", (L, 3 * C)), ("attprojw", (L, C, C)),
+              ("attprojb", (L, C)), ("ln2w", (L, C)), ("ln2b", (L, C)), ("fcw", (L, 4 * C, C)),
+              ("fcb", (L, 4 * C)), ("fcprojw", (L, C, 4 * C)), ("fcprojb", (L, C)),
+              ("lnfw", (C,)), ("lnfb", (C,))]
+    out = []
+    for k, (name, shape) in enumerate(shapes):
+        n = int(np.prod(shape))
+        # multiples of 1/128 below 2^5: exact in bf16 (8 significant bits) as well as fp32
+        vals = (k + 1) + (np.arange(n) % 97) / 128.0
+        out.append((name, shape, vals.astype(np.float32).reshape(shape)))
+    return out
+
+
+def _literal_file(path, version):
+    import struct
+    import torch
+    words = [20240326, version, LIT["max_seq_len"], LIT["vocab_size"], LIT["num_layers"],
+             LIT["num_heads"], LIT["channels"], LIT_VP if version != 1 else 0]
+    blob = bytearray(1024)
+    for i, w in enumerate(words):
+        struct.pack_into("<i", blob, 4 * i, w)
+
+    def raw(a):
+        if version == 5:  # bf16 by torch's conversion, not by the package's bit shifting
+            return torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).view(torch.int16) \
+                .numpy().astype("<i2").tobytes()
+        return np.ascontiguousarray(a).astype("<f4").tobytes()
+
+    for name, shape, vals in _literal_tensors():
+        blob += raw(vals)
+        if name == "wte" and version != 1:
+            pad = np.full((LIT_VP - LIT["vocab_size"], LIT["channels"]), -777.0, np.float32)
+            blob += raw(pad)
+    path.write_bytes(bytes(blob))
+
+
+@pytest.mark.parametrize("version", [1, 3, 5])
+def test_literal_layout_header(tmp_path, version):
+    p = tmp_path / "lit.bin"
+    _literal_file(p, version)
+    assert g2.read_checkpoint_config(p) == LIT
+    n = sum(v.size for _, _, v in _literal_tensors())
+    pad = (LIT_VP - LIT["vocab_size"]) * LIT["channels"] if version != 1 else 0
+    assert p.stat().st_size == 1024 + (2 if version == 5 else 4) * (n + pad)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("version", [1, 3, 5])
+def test_literal_layout_loads_every_tensor_in_place(tmp_path, version):
+    p = tmp_path / "lit.bin"
+    _literal_file(p, version)
+    m = g2.GPT2.from_checkpoint(p)
+    try:
+        flat = m.params_tensor().cpu().numpy()
+        off = 0
+        for name, shape, vals in _literal_tensors():
+            got = flat[off:off + vals.size].reshape(shape)
+            assert np.array_equal(got, vals), f"{name} (version {version})"
+            off += vals.size
+        assert off == flat.size == m.num_parameters
+    finally:
+        m.close()
