@@ -106,8 +106,7 @@ LIT_VP = 256
 
 
 def _literal_tensors():
-    """(name, shape, values) in file order; tensor k holds k + 1 + (flat index mod 251) / 256,
-    all exactly representable in bf16-free fp32 and distinct between tensors."""
+    """(name, shape, values) in file order; tensor k holds ((13 k + flat index) mod 251) - 125."""
     maxT, V, L, C = LIT["max_seq_len"], LIT["vocab_size"], LIT["num_layers"], LIT["channels"]
     shapes = [("wte", (V, C)), ("wpe", (maxT, C)), ("ln1w", (L, C)), ("ln1b", (L, C)),
               ("qkvw", (L, 3 * C, C)), ("qkvb", (L, 3 * C)), ("attprojw", (L, C, C)),
@@ -117,8 +116,9 @@ def _literal_tensors():
     out = []
     for k, (name, shape) in enumerate(shapes):
         n = int(np.prod(shape))
-        # multiples of 1/128 below 2^5: exact in bf16 (8 significant bits) as well as fp32
-        vals = (k + 1) + (np.arange(n) % 97) / 128.0
+        # integers of at most 8 significant bits: exact in bf16 as well as in fp32; the phase
+        # 13 k makes a tensor read from a neighbour's offset differ at every element
+        vals = ((13 * k + np.arange(n)) % 251) - 125.0
         out.append((name, shape, vals.astype(np.float32).reshape(shape)))
     return out
 
