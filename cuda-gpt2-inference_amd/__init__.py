@@ -43,6 +43,7 @@ EXPORTS = (
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
     "matmul_forward_argmax_workspace", "matmul_forward_argmax_status",
+    "matmul_forward_argmax_noalloc_status",
     "gpt2_checkpoint_read_config", "gpt2_build_from_checkpoint",
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
@@ -163,6 +164,8 @@ def lib() -> ctypes.CDLL:
         L.matmul_forward_argmax_workspace.restype = cz
         L.matmul_forward_argmax_status.argtypes = [vp, vp, cz, vp, vp, vp, ci, ci, ci, ci]
         L.matmul_forward_argmax_status.restype = ci
+        L.matmul_forward_argmax_noalloc_status.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci]
+        L.matmul_forward_argmax_noalloc_status.restype = ci
         L.gpt2_forward_profiled_status.argtypes = [vp, vp, ci, ci, ctypes.POINTER(ctypes.c_float)]
         L.gpt2_forward_profiled_status.restype = ci
         L.gpt2_logits.argtypes, L.gpt2_logits.restype = [vp], vp
@@ -280,6 +283,17 @@ def matmul_forward_argmax(ids, inp, weight, bias, B, T, C, OC, workspace=None):
     _check(lib().matmul_forward_argmax_status(_i32(ids), workspace.data_ptr(), workspace.numel(),
                                               _f32(inp), _f32(weight), _f32(bias), B, T, C, OC),
            "matmul_forward_argmax")
+
+
+ARGMAX_NOALLOC_BYTES = 33 << 20  # GPT2HIP_ARGMAX_NOALLOC_BYTES
+
+
+def matmul_forward_argmax_noalloc(ids, inp, weight, bias, B, T, C, OC):
+    """matmul_forward_argmax with the pairs in the library's static device array: no
+    allocation, no workspace argument; shapes beyond ARGMAX_NOALLOC_BYTES of pairs raise."""
+    _check(lib().matmul_forward_argmax_noalloc_status(_i32(ids), _f32(inp), _f32(weight),
+                                                      _f32(bias), B, T, C, OC),
+           "matmul_forward_argmax_noalloc")
 
 
 def set_stream(stream) -> None:

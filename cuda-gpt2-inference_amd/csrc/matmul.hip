@@ -40,6 +40,7 @@
 // with N(0,1) operands and at 2.25-2.35 GHz with all-zero operands, i.e. the chip's
 // power management, not the instruction stream, sets the distance to the 2.4 GHz peak.
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -1175,6 +1176,64 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
   return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu);
 }
 
+// ---- lm-head + argmax -------------------------------------------------------------------
+static int argmax_dispatch(int* ids, void* workspace, size_t workspace_bytes, const float* inp,
+                           const float* weight, const float* bias, int B, int T, int C, int OC) {
+  if (B < 0 || T < 0 || C < 1 || OC < 1)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
+  const long long M64 = (long long)B * T;
+  if (M64 > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: B*T too large");
+  const int M = (int)M64;
+  if (M == 0) return GPT2HIP_OK;
+  if (!ids || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: null pointer");
+  if (C % BK != 0 || !aligned16(inp) || !aligned16(weight) ||
+      (long long)C * 192 * 4 >= (1LL << 31)) {
+    hipLaunchKernelGGL(matmul_argmax_generic_kernel, dim3((unsigned)M), dim3(256), 0, stream(), ids, inp,
+                       weight, bias, C, OC);
+    G2_LAUNCH_CHECK("matmul_forward_argmax");
+    return GPT2HIP_OK;
+  }
+  const size_t need = matmul_forward_argmax_workspace(B, T, OC);
+  if (!workspace || workspace_bytes < need)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: workspace of %zu bytes, need %zu",
+                workspace_bytes, need);
+  const long long tiles = (long long)((M + 127) / 128) * ((OC + 191) / 192);
+  if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: too many tiles");
+  float* pair_val = static_cast<float*>(workspace);
+  int* pair_idx = reinterpret_cast<int*>(pair_val + need / 8);
+  if (tiles >= 16 * 256)
+    return launch_dma_argmax<2>(ids, pair_val, pair_idx, inp, weight, bias, M, C, OC);
+  return launch_dma_argmax<4>(ids, pair_val, pair_idx, inp, weight, bias, M, C, OC);
+}
+
+// The (value, column) pairs of matmul_forward_argmax_noalloc: 33 MiB of device memory that
+// every GPU the library runs on holds from the moment its code is loaded there until the
+// process ends (8192 rows x 524 pairs x 8 bytes, the lm-head of GPT-2 at B*T = 8192).  Every
+// pair a launch reads is written by the same launch first, so nothing needs clearing between
+// calls; two calls that overlap on one GPU (different streams) share the array and race.
+static __device__ __align__(256) unsigned char scratch[GPT2HIP_ARGMAX_NOALLOC_BYTES];
+
+// The array's address on the current device.  `scratch` itself is only a host-side handle:
+// each device has its own copy at its own address, looked up once per device.
+static int scratch_address(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static void* address[kMaxDevices];  // zero-initialised
+  int dev = 0;
+  G2_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_argmax_noalloc: device %d out of range", dev);
+  std::lock_guard<std::mutex> hold(lock);
+  if (!address[dev]) {
+    void* p = nullptr;
+    G2_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(GPT2HIP_EHIP, "matmul_forward_argmax_noalloc: no address for the scratch array");
+    address[dev] = p;
+  }
+  *out = address[dev];
+  return GPT2HIP_OK;
+}
+
 }  // namespace g2
 
 extern "C" {
@@ -1211,32 +1270,21 @@ size_t matmul_forward_argmax_workspace(int B, int T, int OC) {
 int matmul_forward_argmax_status(int* ids, void* workspace, size_t workspace_bytes, const float* inp,
                                  const float* weight, const float* bias, int B, int T, int C,
                                  int OC) {
+  return g2::argmax_dispatch(ids, workspace, workspace_bytes, inp, weight, bias, B, T, C, OC);
+}
+
+int matmul_forward_argmax_noalloc_status(int* ids, const float* inp, const float* weight,
+                                         const float* bias, int B, int T, int C, int OC) {
   using namespace g2;
-  if (B < 0 || T < 0 || C < 1 || OC < 1)
-    return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
-  const long long M64 = (long long)B * T;
-  if (M64 > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: B*T too large");
-  const int M = (int)M64;
-  if (M == 0) return GPT2HIP_OK;
-  if (!ids || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: null pointer");
-  if (C % BK != 0 || !aligned16(inp) || !aligned16(weight) ||
-      (long long)C * 192 * 4 >= (1LL << 31)) {
-    hipLaunchKernelGGL(matmul_argmax_generic_kernel, dim3((unsigned)M), dim3(256), 0, stream(), ids, inp,
-                       weight, bias, C, OC);
-    G2_LAUNCH_CHECK("matmul_forward_argmax");
-    return GPT2HIP_OK;
-  }
   const size_t need = matmul_forward_argmax_workspace(B, T, OC);
-  if (!workspace || workspace_bytes < need)
-    return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: workspace of %zu bytes, need %zu",
-                workspace_bytes, need);
-  const long long tiles = (long long)((M + 127) / 128) * ((OC + 191) / 192);
-  if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward_argmax: too many tiles");
-  float* pair_val = static_cast<float*>(workspace);
-  int* pair_idx = reinterpret_cast<int*>(pair_val + need / 8);
-  if (tiles >= 16 * 256)
-    return launch_dma_argmax<2>(ids, pair_val, pair_idx, inp, weight, bias, M, C, OC);
-  return launch_dma_argmax<4>(ids, pair_val, pair_idx, inp, weight, bias, M, C, OC);
+  if (need > sizeof(scratch))
+    return fail(GPT2HIP_EINVAL,
+                "matmul_forward_argmax_noalloc: B*T=%lld, OC=%d needs %zu bytes of pairs, the "
+                "library's static scratch array holds %zu",
+                (long long)B * T, OC, need, sizeof(scratch));
+  void* ptr = nullptr;
+  if (int rc = scratch_address(&ptr)) return rc;
+  return argmax_dispatch(ids, ptr, sizeof(scratch), inp, weight, bias, B, T, C, OC);
 }
 
 int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,

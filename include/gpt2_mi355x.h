@@ -131,6 +131,20 @@ int matmul_forward_argmax_status(int* ids, void* workspace, size_t workspace_byt
                                  const float* weight, const float* bias, int B, int T, int C,
                                  int OC);
 
+/* matmul_forward_argmax for callers that cannot allocate or hand over a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The (value, column) pairs go to a static array of
+ * GPT2HIP_ARGMAX_NOALLOC_BYTES bytes of device memory inside the library (every GPU the
+ * library runs on holds it until the process ends); the call allocates and frees nothing.
+ * Shapes whose pairs need more (matmul_forward_argmax_workspace(B, T, OC) bytes; the limit
+ * covers B*T = 8192 rows at OC = 50257..50304) are rejected with GPT2HIP_EINVAL.  Results equal
+ * matmul_forward_argmax_status bit for bit.  All calls on one GPU share the array: calls
+ * that overlap on one GPU (different streams or threads) race.  The first call on a device
+ * looks the array's address up (no allocation, but make it outside graph capture). */
+#define GPT2HIP_ARGMAX_NOALLOC_BYTES (33u << 20)
+int matmul_forward_argmax_noalloc_status(int* ids, const float* inp, const float* weight,
+                                         const float* bias, int B, int T, int C, int OC);
+
 /* ---- whole model: the gpt2_forward driver (llm.c train_gpt2_fp32.cu's
  * gpt2_forward, which the reference plugs its kernels into, README.md:19;
  * dataflow in reference images/gpt2/gpt2_flow.png). ---- */
