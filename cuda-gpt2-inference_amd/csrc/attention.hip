@@ -4,47 +4,32 @@
 // on the fp32 matrix cores.  The T x T scores never leave registers.
 //
 // Shape of the computation (head size 64).  A workgroup of 4 waves owns 64
-// consecutive queries of one (batch, head): two groups of 32 queries, each shared
-// by a PAIR of waves that split the keys between them.  Keys and values go from
-// global memory straight into LDS (global_load_lds_dwordx4, two buffers of 64
-// keys, one barrier per tile); of every tile the first wave of a pair takes the
-// first 32 keys and the second wave the last 32, each with its own running
-// maximum, sum and output, and the two partial results are merged once at the
-// end.  Splitting keys rather than queries keeps the four waves of a workgroup
-// equally busy under the causal mask (they differ by at most one sub-tile, on the
-// diagonal), which a split by queries does not: with 128 queries per workgroup and
-// one group per wave, non-causal attention ran at 80 % of the matrix peak and
-// causal attention at 60 %.
+// consecutive queries of one (batch, head) as two groups of 32, each shared by a
+// PAIR of waves that split the keys between them (P = 2), or -- when that would
+// leave compute units without work -- one group of 32 queries split four ways (P = 4).
+// A wave takes every P-th sub-tile of 32 keys, with its own running maximum, sum
+// and output; the partial results of a group are merged once at the end.  Splitting
+// keys rather than queries keeps the waves of a workgroup equally busy under the
+// causal mask (they differ by at most one sub-tile, on the diagonal), which a split
+// by queries does not: with 128 queries per workgroup and one group per wave,
+// non-causal attention ran at 80 % of the matrix peak and causal attention at 60 %.
 //
-// Per sub-tile a wave computes, with v_mfma_f32_32x32x2_f32,
-//     S^T (32 keys x 32 queries) = K_sub (32 x 64) . Q^T (64 x 32)
-// so that lane l owns query l%32 and holds 16 of that query's 32 scores
-// (keys 8*(v/4) + 4*(l/32) + v%4, v = 0..15); lane l^32 holds the other 16.
-// Row maxima and sums are therefore register reductions plus one exchange
-// with lane l^32 (v_permlane32_swap).  The probabilities are then used IN PLACE
-// as the B operand of
-//     O^T (64 x 32 queries) += V_sub^T (64 x 32 keys) . P^T (32 keys x 32 queries)
-// because the accumulator layout of S^T is exactly a valid B-operand layout
-// once the k index of each MFMA is read as "key 8*(v/4)+v%4 for lanes 0..31,
-// that key + 4 for lanes 32..63"; the matching V rows are picked by address.
-// (The reference bounces P through shared memory for this step,
-// 2_flash_attention.cuh:227-240.)
+// The waves of a workgroup share nothing inside the loop, so there is no barrier in
+// it.  A wave's K sub-tile (8 KiB) goes from global memory straight into the wave's
+// own LDS region (buffer_load ... lds); as soon as the wave has read it into
+// registers it requests the next one into the same region, which then has a whole
+// sub-tile of matrix work to arrive.  V needs no transposition (a lane wants two
+// neighbouring features of one key: a wave load is two 256-byte rows) and goes
+// straight from global memory to registers, requested before the scores and used
+// after the softmax.  34 KiB of LDS and 160 registers per lane leave room for three
+// workgroups per compute unit, which is what hides a workgroup's start (first
+// loads) and end (merge, stores) behind the matrix work of the others: the earlier
+// form (keys and values of 64-key tiles shared through 64 KiB of LDS by the four
+// waves, one barrier per tile, two workgroups per compute unit) ran the benchmark
+// shape B=8, T=1024, NH=12 in 128.8 us where this one takes 121.0 in the same harness.
+// Addresses are buffer addresses (scalar base + scalar row offset + a fixed lane offset):
+// no vector address arithmetic in the loop, and rows at or past T read as zeros.
 //
-// Q is held in registers for the whole kernel in the same k-permuted form the
-// GEMM uses (lane half h holds hs = 8g+4h..+3 of group g), K tiles are stored
-// with the same XOR chunk swizzle, and V rows are read as 64-bit pairs so that
-// accumulator a (0/1) of lane l, register v holds output feature
-// 16*(v/4) + 8*(l/32) + 2*(v%4) + a: eight consecutive floats per v/4, stored
-// as two 128-bit writes.
-//
-// Every VALU instruction takes issue time from the matrix pipe on this chip, so
-// the softmax is kept lean: hardware exp2 on a fused multiply-add, and a LAZY
-// running maximum — the shift m only moves when some score exceeds it by more
-// than 2^8 after scaling, so the rescaling of O and of the running sum is a rare,
-// wave-uniform branch.  Softmax is invariant to the shift, so this is exact;
-// probabilities are merely allowed to reach 2^8 instead of 1 before normalisation.
-// (The branch is taken per group of 32 queries, so the ROUNDING of a query's result
-// can depend on the other queries of its group; its value cannot.)
 #include <type_traits>
 
 #include "common.hpp"
@@ -52,17 +37,15 @@
 namespace g2 {
 
 constexpr int HS = 64;          // head size this kernel is built for
-constexpr int BQ = 64;          // queries per workgroup (2 groups of 32, 2 waves each)
-constexpr int BKV = 64;         // keys per LDS tile
-constexpr int KV_CH = HS / 4;   // 16-byte chunks per K/V row
 constexpr int ATT_THREADS = 256;
 constexpr int ATT_WAVES = ATT_THREADS / kWave;
-constexpr int KV_TILE_BYTES = BKV * HS * 4;                 // 16 KiB per tensor per tile
-constexpr int KV_DMA_PER = 2 * (KV_TILE_BYTES / 1024) / ATT_WAVES;  // K+V DMAs per wave and tile = 8
+constexpr int K_SUB_BYTES = 32 * HS * 4;          // one sub-tile of 32 keys: 8 KiB
+constexpr int WAVE_LDS_BYTES = 34 * kWave * 4;    // a wave's region: its K sub-tile, later its parked partial state
 constexpr float LAZY_LOG2 = 8.0f;  // allowed growth of 2^x above the current shift
 
 typedef __attribute__((address_space(3))) void lds_void_t;
-typedef const __attribute__((address_space(1))) void glb_void_t;
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 // Exchange between lanes l and l^32: v_permlane32_swap swaps lanes 32..63 of its
 // first operand with lanes 0..31 of its second.  Fed two copies of x it leaves
@@ -85,12 +68,15 @@ __device__ __forceinline__ float pair_sum(float x) {
   return lo + hi;
 }
 
-__global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
-    float* __restrict__ out, const float* __restrict__ qkv, int T, int NH, int nqt,
-    float scale_log2e) {
-  // [buffer][K tile | V tile]
-  __shared__ f32x4 kv_lds[2][2 * BKV * KV_CH];
-  char* const lds_bytes = reinterpret_cast<char*>(&kv_lds[0][0]);
+// P = waves that split the keys of one group of 32 queries; a workgroup of 4 waves holds
+// 4 / P such groups.
+template <int P>
+__global__ __launch_bounds__(ATT_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3)))
+void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ qkv, int T, int NH,
+                            int nqb, float scale_log2e) {
+  constexpr int QG = ATT_WAVES / P;  // query groups per workgroup
+  constexpr int BQ = 32 * QG;        // queries per workgroup
+  __shared__ __attribute__((aligned(16))) char lds_all[ATT_WAVES * WAVE_LDS_BYTES];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -98,76 +84,56 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
   const int h32 = lane >> 5;
   const int l32 = lane & 31;
 
-  // heaviest query tiles (most keys) are launched first
+  // heaviest query blocks (most keys) are launched first
   const int bid = blockIdx.x;
-  const int per_tile = gridDim.x / nqt;  // = B*NH
-  const int qtile = nqt - 1 - bid / per_tile;
-  const int bh = bid % per_tile;
+  const int per_block = gridDim.x / nqb;  // = B*NH
+  const int qblock = nqb - 1 - bid / per_block;
+  const int bh = bid % per_block;
   const int b = bh / NH, head = bh % NH;
 
   const int C = NH * HS;
-  const size_t row_stride = (size_t)3 * C;
-  const float* base = qkv + (size_t)b * T * row_stride + head * HS;
+  const int row_bytes = 3 * C * 4;
+  const int qgroup = wave / P;        // which 32 queries of the workgroup
+  const int part = wave % P;          // which sub-tiles of 32 keys: part, part + P, ...
+  const int qw = qblock * BQ + qgroup * 32;  // first query of this wave
+  const int myq = qw + l32;                  // this lane's query
+  const int diag = qw >> 5;                  // the sub-tile that holds the diagonal; the last one needed
+  const bool live = qw < T;                  // a group entirely past T has nothing to do
 
-  const int q0 = qtile * BQ;          // first query of the workgroup
-  const int qgroup = wave >> 1;       // which 32 queries
-  const int khalf = wave & 1;         // which 32 keys of every 64-key tile
-  const int qw = q0 + qgroup * 32;    // first query of this wave
-  const int myq = qw + l32;           // this lane's query
-  const int kv_end = min(T, q0 + BQ); // keys the workgroup needs: [0, kv_end)
-  const int ntile = (kv_end + BKV - 1) / BKV;
+  // One sequence's packed rows as a buffer: offsets are 32-bit, and rows at or past T read
+  // as zeros (keys there only meet masked or unstored queries).
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(qkv) + (size_t)b * T * 3 * C, 0, T * row_bytes, 0x00020000);
+  const int q_col = head * (HS * 4), k_col = q_col + C * 4, v_col = q_col + 2 * C * 4;
+
+  char* const my_lds = lds_all + wave * WAVE_LDS_BYTES;
+
+  // ---- K sub-tile: global -> LDS by DMA, 8 instructions of 4 rows x 256 bytes --------
+  // Lane l lands at slot l of the instruction's KiB: row l/16, chunk position l%16, and
+  // fetches logical chunk (l%16) ^ (row & 7) (the swizzle is applied on the global side).
+  // row & 7 = 4*(i&1) + l/16 for instruction i, so two lane offsets cover all eight.
+  const int dma_lane[2] = {(lane >> 4) * row_bytes + (((lane & 15) ^ (lane >> 4)) << 4),
+                           (lane >> 4) * row_bytes + (((lane & 15) ^ (4 + (lane >> 4))) << 4)};
+  auto dma_k = [&](int sub) {
+    const int s0 = sub * 32 * row_bytes + k_col;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_t*)(my_lds + i * 1024), 16, dma_lane[i & 1],
+                                               s0 + 4 * i * row_bytes, 0, 0);
+  };
+
+  int sub = part;
+  if (live && sub <= diag) dma_k(sub);
 
   // ---- Q in registers: qreg[g] = Q[myq][8g+4h .. +3] --------------------
   f32x4 qreg[8];
   {
-    const int qr = min(myq, T - 1);  // clamp: out-of-range queries compute garbage, never stored
-    const f32x4* qp = reinterpret_cast<const f32x4*>(base + (size_t)qr * row_stride);
+    const int qv = l32 * row_bytes + h32 * 16;
+    const int qs = qw * row_bytes + q_col;
 #pragma unroll
-    for (int g = 0; g < 8; g++) qreg[g] = qp[2 * g + h32];
+    for (int g = 0; g < 8; g++)
+      qreg[g] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, qv, qs + g * 32, 0));
   }
-
-  // ---- K/V LDS-DMA: one instruction moves 4 rows of 256 bytes ------------------
-  // DMA j of this wave: group gi = wave*KV_DMA_PER + j of the tile's 32 groups
-  // (0..15: K rows 4*gi.., 16..31: V rows).  Lane l lands at LDS slot l of the group:
-  // row l/16, chunk position l%16; for K it fetches logical chunk (l%16) ^ (row & 7).
-  // An address is a wave-uniform base (the tile's first K row, moved on with scalar
-  // adds) plus a fixed 32-bit per-lane offset.  Only a last, partial tile (T % 64 != 0)
-  // needs per-lane work: keys at or past T are clamped to T-1 there; they only ever
-  // meet queries < key, i.e. they are masked, or queries >= T, which are not stored.
-  const char* const kv_base = reinterpret_cast<const char*>(base + C);  // K; V is C floats on
-  const unsigned row_bytes = (unsigned)(row_stride * 4);
-  int dma_row[KV_DMA_PER];       // row inside the tile
-  unsigned dma_col[KV_DMA_PER];  // byte offset inside the (K|V) row, V's includes +C floats
-  unsigned dma_off[KV_DMA_PER];  // dma_row * row_bytes + dma_col
-#pragma unroll
-  for (int j = 0; j < KV_DMA_PER; j++) {
-    const int gi = wave * KV_DMA_PER + j;
-    const bool is_v = gi >= 16;
-    const int row = 4 * (gi & 15) + (lane >> 4);
-    const int c = is_v ? (lane & 15) : ((lane & 15) ^ (row & 7));
-    dma_row[j] = row;
-    dma_col[j] = (unsigned)(c * 16 + (is_v ? C * 4 : 0));
-    dma_off[j] = (unsigned)row * row_bytes + dma_col[j];
-  }
-  auto dma_tile = [&](int tile, int buf) {
-    const char* tile_base = kv_base + (size_t)tile * BKV * row_bytes;
-    char* const dst = lds_bytes + buf * (2 * KV_TILE_BYTES) + wave * (KV_DMA_PER * 1024);
-    if ((tile + 1) * BKV <= T) {
-      asm volatile("" : "+s"(tile_base));  // keep "scalar base + lane offset" intact for selection
-#pragma unroll
-      for (int j = 0; j < KV_DMA_PER; j++)
-        __builtin_amdgcn_global_load_lds((glb_void_t*)(tile_base + dma_off[j]),
-                                         (lds_void_t*)(dst + j * 1024), 16, 0, 0);
-    } else {
-#pragma unroll
-      for (int j = 0; j < KV_DMA_PER; j++) {
-        const int key = min(tile * BKV + dma_row[j], T - 1);
-        __builtin_amdgcn_global_load_lds(
-            (glb_void_t*)(kv_base + (size_t)key * row_bytes + dma_col[j]),
-            (lds_void_t*)(dst + j * 1024), 16, 0, 0);
-      }
-    }
-  };
 
   f32x16 o0, o1;
 #pragma unroll
@@ -180,127 +146,97 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
   float l_run = 0.f;         // this lane's share of the running denominator
   const float lazy_raw = LAZY_LOG2 / scale_log2e;
 
-  // LDS read addresses (bytes, inside buffer 0, sub-tile 0); buffer and sub-tile are
-  // immediate offsets of the read instructions.
-  int k_addr[8];
+  // LDS read addresses of the K operand: row l32, chunk (2g+h) ^ (l32 & 7); chunks of g and
+  // g + 4 are 128 bytes apart
+  const char* k_addr[4];
 #pragma unroll
-  for (int g = 0; g < 8; g++) k_addr[g] = (l32 * KV_CH + ((2 * g + h32) ^ (lane & 7))) * 16;
-  const int v_addr = KV_TILE_BYTES + (4 * h32) * (HS * 4) + l32 * 8;
+  for (int g = 0; g < 4; g++) k_addr[g] = my_lds + (l32 * 16 + ((2 * g + h32) ^ (lane & 7))) * 16;
+  // V straight from global memory: register v pairs with key 8*(v/4) + 4*h32 + v%4 of the
+  // sub-tile, this lane's two features are 2*l32, 2*l32+1
+  const int v_lane = 4 * h32 * row_bytes + l32 * 8;
 
-  // Operand registers of one sub-tile: K as eight 16-byte chunks (A operand of the
-  // score MFMAs), V as sixteen 8-byte pairs (A operand of the output MFMAs).
-  struct Operands {
-    f32x4 k[8];
-    f32x2 v[16];
-  };
-  // All LDS reads of a sub-tile are issued in one batch, well before their first use:
-  // V is read before the score MFMAs that precede its use, and the next sub-tile's K
-  // before the output MFMAs of the current one.
-  auto read_k = [&](Operands& op, int off) {
+  if (live) {
+    for (; sub <= diag; sub += P) {
+      const int k0 = sub * 32;
+      // K of this sub-tile has landed (requested one sub-tile ago)
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      f32x4 kreg[8];
 #pragma unroll
-    for (int g = 0; g < 8; g++)
-      op.k[g] = *reinterpret_cast<const f32x4*>(lds_bytes + k_addr[g] + off);
-  };
-  auto read_v = [&](Operands& op, int off) {
+      for (int g = 0; g < 8; g++)
+        kreg[g] = *reinterpret_cast<const f32x4*>(k_addr[g & 3] + (g >> 2) * 128);
+      // V of this sub-tile: needed after the scores and the softmax
+      f32x2 vreg[16];
+      {
+        const int vs = k0 * row_bytes + v_col;
 #pragma unroll
-    for (int v = 0; v < 16; v++)
-      op.v[v] = *reinterpret_cast<const f32x2*>(lds_bytes + v_addr +
-                                                (off + (8 * (v >> 2) + (v & 3)) * (HS * 4)));
-  };
+        for (int v = 0; v < 16; v++)
+          vreg[v] = __builtin_bit_cast(
+              f32x2, __builtin_amdgcn_raw_buffer_load_b64(rsrc, v_lane, vs + (8 * (v >> 2) + (v & 3)) * row_bytes, 0));
+      }
+      // the K region is free once its reads have returned: request the next sub-tile
+      if (sub + P <= diag) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        dma_k(sub + P);
+      }
 
-  // Scores, lazy online softmax and output update of one sub-tile of 32 keys.
-  auto sub_tile = [&](int k0, const Operands& op, auto&& before_output) {
-    // S^T = K_sub . Q^T
-    f32x16 s;
+      // S^T = K_sub . Q^T
+      f32x16 s;
 #pragma unroll
-    for (int v = 0; v < 16; v++) s[v] = 0.f;
+      for (int v = 0; v < 16; v++) s[v] = 0.f;
 #pragma unroll
-    for (int g = 0; g < 8; g++)
+      for (int g = 0; g < 8; g++)
 #pragma unroll
-      for (int e = 0; e < 4; e++)
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(op.k[g][e], qreg[g][e], s, 0, 0, 0);
+        for (int e = 0; e < 4; e++)
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[g][e], qreg[g][e], s, 0, 0, 0);
 
-    // causal mask on the diagonal sub-tile
-    if (k0 + 31 > qw) {
+      // causal mask on the diagonal sub-tile (keys at or past T are beyond every stored query)
+      if (sub == diag) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int key = k0 + 8 * (v >> 2) + 4 * h32 + (v & 3);
+          if (key > myq) s[v] = -INFINITY;
+        }
+      }
+
+      // lazy online softmax for this lane's query
+      float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+      for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
+      mx = pair_max(fmaxf(mx, s[15]));  // finite: key k0 <= every query of the wave
+      if (__builtin_amdgcn_ballot_w64(mx > m_used + lazy_raw) != 0) {
+        const float m_new = fmaxf(m_used, mx);
+        const float alpha = __builtin_amdgcn_exp2f((m_used - m_new) * scale_log2e);  // 0 at first
+        m_used = m_new;
+        mc = m_new * scale_log2e;
+        l_run *= alpha;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          o0[v] *= alpha;
+          o1[v] *= alpha;
+        }
+      }
+      float psum = 0.f;
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const int key = k0 + 8 * (v >> 2) + 4 * h32 + (v & 3);
-        if (key > myq) s[v] = -INFINITY;
+        s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], scale_log2e, -mc));
+        psum += s[v];
       }
-    }
+      l_run += psum;
 
-    // lazy online softmax for this lane's query
-    float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
-#pragma unroll
-    for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
-    mx = pair_max(fmaxf(mx, s[15]));  // finite: key k0 <= every query of the wave
-    if (__builtin_amdgcn_ballot_w64(mx > m_used + lazy_raw) != 0) {
-      const float m_new = fmaxf(m_used, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_used - m_new) * scale_log2e);  // 0 at first
-      m_used = m_new;
-      mc = m_new * scale_log2e;
-      l_run *= alpha;
+      // O^T += V_sub^T . P^T
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        o0[v] *= alpha;
-        o1[v] *= alpha;
+        o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[v].x, s[v], o0, 0, 0, 0);
+        o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[v].y, s[v], o1, 0, 0, 0);
       }
     }
-    float psum = 0.f;
-#pragma unroll
-    for (int v = 0; v < 16; v++) {
-      s[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], scale_log2e, -mc));
-      psum += s[v];
-    }
-    l_run += psum;
-
-    before_output();
-
-    // O^T += V_sub^T . P^T : register v pairs with key 8*(v/4) + 4*h32 + v%4
-#pragma unroll
-    for (int v = 0; v < 16; v++) {
-      o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(op.v[v].x, s[v], o0, 0, 0, 0);
-      o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(op.v[v].y, s[v], o1, 0, 0, 0);
-    }
-  };
-
-  // One tile of 64 keys out of buffer BUF (a compile-time constant, so that every LDS
-  // address is register + immediate).
-  auto tile_body = [&](int tile, auto buf_tag) {
-    constexpr int BUF = decltype(buf_tag)::value;
-    constexpr int kbuf = BUF * (2 * KV_TILE_BYTES);
-    constexpr int sub1 = 32 * (HS * 4);
-    // the other buffer was last read before the barrier that ended the previous tile
-    if (tile + 1 < ntile) dma_tile(tile + 1, BUF ^ 1);
-
-    // this wave's 32 keys of the tile; wave-uniform: do they reach down to the diagonal?
-    const int k0 = tile * BKV + khalf * 32;
-    if (k0 <= qw + 31 && k0 < T) {
-      Operands a;
-      read_k(a, kbuf + khalf * sub1);
-      read_v(a, kbuf + khalf * sub1);
-      sub_tile(k0, a, []() {});
-    }
-
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): my DMAs of the next tile have landed
-    __syncthreads();
-  };
-
-  dma_tile(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  __syncthreads();
-  int tile = 0;
-  for (; tile + 1 < ntile; tile += 2) {
-    tile_body(tile, std::integral_constant<int, 0>{});
-    tile_body(tile + 1, std::integral_constant<int, 1>{});
   }
-  if (tile < ntile) tile_body(tile, std::integral_constant<int, 0>{});
 
-  // ---- merge the two key halves of each query group --------------------------
-  // The K/V buffers are idle after the loop's last barrier; the second wave of each
-  // pair parks its partial state there, one float per (register, lane).
-  float* const park = reinterpret_cast<float*>(lds_bytes) + qgroup * (35 * kWave) + lane;
-  if (khalf == 1) {
+  // ---- merge the P key parts of each query group --------------------------
+  // Every wave's K region is idle once its own loop has ended; parts 1 .. P-1 park their
+  // partial state there, one float per (register, lane).
+  float* const park = reinterpret_cast<float*>(my_lds) + lane;
+  if (part != 0 && live && part <= diag) {
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       park[v * kWave] = o0[v];
@@ -310,17 +246,26 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_flash_kernel(
     park[33 * kWave] = l_run;
   }
   __syncthreads();
-  if (khalf == 0) {
-    const float m1 = park[32 * kWave], l1 = park[33 * kWave];
-    const float m = fmaxf(m_used, m1);  // m_used is finite: key 0 is visible to every query
-    const float a0 = __builtin_amdgcn_exp2f((m_used - m) * scale_log2e);
-    const float a1 = __builtin_amdgcn_exp2f((m1 - m) * scale_log2e);  // 0 if that half saw no key
+  if (part == 0 && live) {
+    // m_used is finite: key 0 is visible to every query, and sub-tile 0 belongs to part 0
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-      o0[v] = o0[v] * a0 + park[v * kWave] * a1;
-      o1[v] = o1[v] * a0 + park[(16 + v) * kWave] * a1;
+    for (int p = 1; p < P; p++) {
+      if (p <= diag) {
+        const float* other = reinterpret_cast<const float*>(lds_all + (wave + p) * WAVE_LDS_BYTES) + lane;
+        const float m1 = other[32 * kWave], l1 = other[33 * kWave];
+        const float m = fmaxf(m_used, m1);
+        const float a0 = __builtin_amdgcn_exp2f((m_used - m) * scale_log2e);
+        const float a1 = __builtin_amdgcn_exp2f((m1 - m) * scale_log2e);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          o0[v] = o0[v] * a0 + other[v * kWave] * a1;
+          o1[v] = o1[v] * a0 + other[(16 + v) * kWave] * a1;
+        }
+        l_run = l_run * a0 + l1 * a1;
+        m_used = m;
+      }
     }
-    const float inv = 1.0f / pair_sum(l_run * a0 + l1 * a1);
+    const float inv = 1.0f / pair_sum(l_run);
     if (myq < T) {
       float* op = out + ((size_t)b * T + myq) * C + head * HS + 8 * h32;
 #pragma unroll
@@ -656,13 +601,22 @@ int attention_forward_status(float* out, float* qkvr, float* att, const float* i
   if (B == 0 || T == 0) return GPT2HIP_OK;
   if (!out || !inp) return fail(GPT2HIP_EINVAL, "attention_forward: null pointer");
   const int hs = C / NH;
-  if (hs == HS && aligned16(inp) && aligned16(out)) {
-    const int nqt = (T + BQ - 1) / BQ;
-    const long long blocks = (long long)nqt * B * NH;
+  if (hs == HS && aligned16(inp) && aligned16(out) && (long long)T * 3 * C * 4 < (1LL << 31)) {
+    // two query groups per workgroup, unless that makes fewer than two workgroups per
+    // compute unit (short sequences, few heads): then one group, keys split four ways
+    const long long wide = (long long)((T + 63) / 64) * B * NH;
+    const int P = wide < 512 ? 4 : 2;
+    const int bq = 32 * (ATT_WAVES / P);
+    const int nqb = (T + bq - 1) / bq;
+    const long long blocks = (long long)nqb * B * NH;
     if (blocks > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "attention_forward: grid too large");
     const float scale_log2e = (1.0f / sqrtf((float)hs)) * 1.4426950408889634f;
-    hipLaunchKernelGGL(attention_flash_kernel, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out,
-                       inp, T, NH, nqt, scale_log2e);
+    if (P == 2)
+      hipLaunchKernelGGL(attention_flash_kernel<2>, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out,
+                         inp, T, NH, nqb, scale_log2e);
+    else
+      hipLaunchKernelGGL(attention_flash_kernel<4>, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out,
+                         inp, T, NH, nqb, scale_log2e);
   } else {
     if (hs > 256) return fail(GPT2HIP_EINVAL, "attention_forward: head size %d > 256", hs);
     const long long waves = (long long)B * NH * T;
