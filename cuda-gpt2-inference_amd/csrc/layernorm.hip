@@ -13,6 +13,22 @@ namespace g2 {
 
 constexpr int kWavesPerBlock = 4;  // 256 threads
 
+// One (N, C) array as a buffer: 128-bit accesses at a 32-bit byte offset, loads non-temporal,
+// stores non-temporal or plain.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+struct Stream {
+  __amdgpu_buffer_rsrc_t rsrc;
+  __device__ __forceinline__ Stream(const float* base, int N, int C)
+      : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)((size_t)N * C * 4), 0x00020000)) {}
+  __device__ __forceinline__ f32x4 load(int byte) const {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte, 0, 2));
+  }
+  template <bool NT>
+  __device__ __forceinline__ void store(int byte, f32x4 v) const {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, byte, 0, NT ? 2 : 0);
+  }
+};
+
 // NV float4 per lane cover C <= 256*NV.  FUSED adds inp2 and stores the sum.  A wave
 // owns ROWS consecutive rows and issues all of their loads before it touches any of
 // them: at N = 8192 four rows per wave (a quarter of the waves, four times the bytes
@@ -28,7 +44,13 @@ constexpr int kWavesPerBlock = 4;  // 256 threads
 // the two arrays every kilobyte.  With streaming stores this moved C = 768 from 17.8 to 16.9 us
 // per launch at N = 8192 (70.6 -> 74.6 % of HBM peak); at C = 1024 with eight rows per wave
 // neither change pays (22.2 us = 75.6 % as it is, 22.4-23.6 us with either or both).
-template <int NV, int ROWS, bool FUSED, bool EXACT, bool NTS, bool BY_STREAM = false>
+// BUF (fused, exact form only): the four big arrays are addressed as buffers (a scalar
+// descriptor and one 32-bit byte offset per lane, the row and chunk as immediates) instead
+// of 64-bit pointers: fewer address instructions ahead of the first load, 17.3 -> 16.8 us
+// at C = 768 (at C = 1024 with eight rows per wave it changes nothing: 22.5 / 22.7 us).
+// Needs N*C*4 < 2^31.
+template <int NV, int ROWS, bool FUSED, bool EXACT, bool NTS, bool BY_STREAM = false,
+          bool BUF = false>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
     float* res_out, float* out, float* __restrict__ mean, float* __restrict__ rstd,
     const float* inp1, const float* inp2, const float* __restrict__ weight,
@@ -39,7 +61,33 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
   const int C4 = C >> 2;
 
   f32x4 v[ROWS][NV];
-  if constexpr (BY_STREAM) {
+  [[maybe_unused]] const int lane_byte = row0 * C * 4 + lane * 16;  // BUF: this lane's first chunk
+  [[maybe_unused]] const Stream X1(inp1, N, C), X2(inp2, N, C), RO(res_out, N, C), O(out, N, C);
+  if constexpr (BUF) {
+    static_assert(FUSED && EXACT, "BUF is a form of the fused kernel without bounds checks");
+    const int row_bytes = C * 4;
+    if constexpr (BY_STREAM) {
+      f32x4 u[ROWS][NV];
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int j = 0; j < NV; j++) v[r][j] = X1.load(lane_byte + r * row_bytes + j * 1024);
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int j = 0; j < NV; j++) u[r][j] = X2.load(lane_byte + r * row_bytes + j * 1024);
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int j = 0; j < NV; j++) v[r][j] += u[r][j];
+    } else {
+#pragma unroll
+      for (int r = 0; r < ROWS; r++)
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+          v[r][j] = X1.load(lane_byte + r * row_bytes + j * 1024) + X2.load(lane_byte + r * row_bytes + j * 1024);
+    }
+  } else if constexpr (BY_STREAM) {
     static_assert(FUSED && EXACT, "BY_STREAM is a form of the fused kernel without bounds checks");
     const f32x4* x1 = reinterpret_cast<const f32x4*>(inp1) + (size_t)row0 * C4 + lane;
     const f32x4* x2 = reinterpret_cast<const f32x4*>(inp2) + (size_t)row0 * C4 + lane;
@@ -90,7 +138,9 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
       for (int j = 0; j < NV; j++) {
         const int c = lane + j * kWave;
         if (EXACT || c < C4) {
-          if (NTS)
+          if constexpr (BUF)
+            RO.template store<NTS>(lane_byte + r * C * 4 + j * 1024, v[r][j]);
+          else if (NTS)
             __builtin_nontemporal_store(v[r][j], ro + c);
           else
             ro[c] = v[r][j];
@@ -131,7 +181,9 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void layernorm_rows_kernel(
       const int c = lane + j * kWave;
       if (EXACT || c < C4) {
         const f32x4 n = (v[r][j] - m) * rs;
-        if (NTS)
+        if constexpr (BUF)
+          O.template store<NTS>(lane_byte + r * C * 4 + j * 1024, n * w4[c] + b4[c]);
+        else if (NTS)
           __builtin_nontemporal_store(n * w4[c] + b4[c], o + c);
         else
           o[c] = n * w4[c] + b4[c];
@@ -208,13 +260,13 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
                      dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, stream(), \
                      res_out, out, mean, rstd, inp1, inp2, weight, bias, N, C)
 #define G2_LN_ROWS(NV)                                              \
-  if (wide && C == 256 * NV && N % 8 == 0) {                        \
+  if (wide && C == 256 * NV && N % 8 == 0 && (long long)N * C * 4 < (1LL << 31)) { \
     if (!FUSED) {                                                   \
       G2_LN(NV, 2, true, true);                                     \
     } else if (NV == 4) {                                           \
       G2_LN(NV, 8, true, false);                                    \
     } else {                                                        \
-      G2_LN(NV, 4, true, true, FUSED);                              \
+      G2_LN(NV, 4, true, true, FUSED, FUSED);                       \
     }                                                               \
   } else if (wide) {                                                \
     G2_LN(NV, 4, false, false);                                     \
