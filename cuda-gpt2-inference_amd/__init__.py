@@ -40,6 +40,7 @@ EXPORTS = (
     "gelu_forward", "gelu_forward_status",
     "matmul_forward", "matmul_forward_status",
     "matmul_forward_gelu", "matmul_forward_gelu_status", "matmul_forward_probe_status",
+    "matmul_forward_tile_shape",
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
     "matmul_forward_argmax_workspace", "matmul_forward_argmax_status",
@@ -133,6 +134,8 @@ def lib() -> ctypes.CDLL:
             f.argtypes, f.restype = args, ci
         L.matmul_forward_probe_status.argtypes = [vp] * 4 + [ci] * 4 + [vp, ci, ctypes.POINTER(ci)]
         L.matmul_forward_probe_status.restype = ci
+        L.matmul_forward_tile_shape.argtypes = [ci] * 4 + [ctypes.POINTER(ci)] * 2
+        L.matmul_forward_tile_shape.restype = ci
         L.gpt2_create.argtypes, L.gpt2_create.restype = [ctypes.POINTER(GPT2Config)], vp
         L.gpt2_destroy.argtypes, L.gpt2_destroy.restype = [vp], None
         L.gpt2_checkpoint_read_config.argtypes = [ctypes.c_char_p, ctypes.POINTER(GPT2Config)]
@@ -262,6 +265,15 @@ def matmul_forward_probe(out, inp, weight, bias, B, T, C, OC):
            "matmul_forward_probe")
     torch.cuda.synchronize()
     return probe[:n.value].cpu().numpy()
+
+
+def matmul_forward_tile_shape(B, T, C, OC):
+    """(rows, columns) of the workgroup tile matmul_forward gives this problem; (0, 0) if it
+    takes a kernel that is not tiled this way.  No GPU needed."""
+    bm, bn = ctypes.c_int(0), ctypes.c_int(0)
+    _check(lib().matmul_forward_tile_shape(B, T, C, OC, ctypes.byref(bm), ctypes.byref(bn)),
+           "matmul_forward_tile_shape")
+    return bm.value, bn.value
 
 
 def attention_forward(out, qkvr, att, inp, B, T, C, NH):

@@ -1049,8 +1049,8 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
   return GPT2HIP_OK;
 }
 
-// LDS-DMA kernel: K % 32 == 0.
-template <int BM, int BN, int WGM, int WGN>
+// LDS-DMA kernel: K % 32 == 0.  The clock-probe form exists for PROBED tile shapes only.
+template <int BM, int BN, int WGM, int WGN, bool PROBED = false>
 static int launch_dma(float* out, const float* inp, const float* weight, const float* bias, int M,
                       int K, int N, bool gelu, unsigned long long* probe = nullptr) {
   constexpr int NT = WGM * WGN * kWave;
@@ -1058,9 +1058,12 @@ static int launch_dma(float* out, const float* inp, const float* weight, const f
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
   const long long tiles = (long long)ntm * ntn;
   if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
-  auto kfn = probe ? matmul_dma_kernel<BM, BN, WGM, WGN, false, true>
-                   : gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true>
-                          : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
+  auto kfn = gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true> : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
+  if constexpr (PROBED) {
+    if (probe) kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, true>;
+  } else if (probe) {
+    return fail(GPT2HIP_EINVAL, "matmul_forward_probe: no probe form of the %dx%d tile", BM, BN);
+  }
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
                      K, N, ntm, ntn, probe, (int*)nullptr);
@@ -1106,6 +1109,54 @@ static int launch_ring(float* out, const float* inp, const float* weight, const 
   return GPT2HIP_OK;
 }
 
+// Tile choice.  A launch of tiles of one shape takes, to within a few per cent over
+// M = 64 .. 8192 at the GPT-2 124M and 350M shapes (fitted per shape to a sweep in which
+// every shape was forced on every problem),
+//     launch + ceil(tiles / 256 CUs) x (a x tile area x K / per-CU MFMA rate + round)
+// where a "round" of one tile per compute unit costs its matrix work (a: the smaller the
+// tile, the more bytes go through LDS per MFMA) plus the part of a tile's first loads and
+// final stores that nothing hides.  The shape with the least predicted time wins: over
+// the sweep its time is within 2.4 % of the best forced shape's (0.13 % on average).  A
+// problem whose tile count is just above a multiple of 256 with the largest tile (124M qkv
+// at M = 4096: 384 tiles of 128x192, two rounds for one and a half rounds of work, 65 % of
+// peak) takes a smaller tile that divides evenly (768 tiles of 128x96, three exact rounds,
+// 85 %).  The clock probe exists for the two largest shapes only.
+struct TileChoice {
+  int index;        // into the candidate list below
+  int bm, bn;
+  long long tiles;
+};
+static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only) {
+  struct Cand { int bm, bn; double a, round_us, launch_us; };
+  // (64x192 and 128x64 were fitted too -- a = 1.033 and 1.042 -- and never won by more than
+  // 0.4 % anywhere in the sweep: not built)
+  const Cand cands[] = {{128, 192, 0.988, 6.42, -2.15}, {128, 128, 1.006, 3.59, -0.11},
+                        {128, 96, 1.017, 1.84, 1.93},   {64, 128, 1.042, 2.08, 1.01},
+                        {64, 64, 1.159, 0.40, 1.88},    {32, 32, 1.398, 0.0, 3.54}};
+  constexpr int kCands = (int)(sizeof(cands) / sizeof(cands[0]));
+  constexpr double kCuFlopsPerUs = 579e3;  // what one compute unit sustains in the 128x192 loop
+  int best = 0;
+  double best_cost = 0;
+  long long best_tiles = 0;
+  for (int i = 0; i < (two_largest_only ? 2 : kCands); i++) {
+    const long long t = (long long)((M + cands[i].bm - 1) / cands[i].bm) *
+                        ((OC + cands[i].bn - 1) / cands[i].bn);
+    Cand c = cands[i];
+    if (i == 4 && t <= 2 * 256) c = Cand{64, 64, 1.190, 0.35, 2.98};  // the ring form of 64x64
+    const double work_us = 2.0 * c.bm * c.bn * (double)C / kCuFlopsPerUs;
+    const double cost = c.launch_us + (double)((t + 255) / 256) * (c.a * work_us + c.round_us);
+    if (i == 0 || cost < best_cost) {
+      best = i;
+      best_cost = cost;
+      best_tiles = t;
+    }
+    // sixteen or more rounds of the largest tile (the lm-head): rounding up to whole
+    // rounds costs at most 3 %, less than any smaller tile loses
+    if (i == 0 && t >= 16 * 256) break;
+  }
+  return TileChoice{best, cands[best].bm, cands[best].bn, best_tiles};
+}
+
 static int matmul_dispatch(float* out, const float* inp, const float* weight, const float* bias,
                            int B, int T, int C, int OC, bool gelu,
                            unsigned long long* probe = nullptr, int* probe_groups = nullptr) {
@@ -1128,48 +1179,34 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
     return skinny_launch(out, inp, weight, bias, nullptr, nullptr, nullptr, M, C, OC, gelu);
   // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
   if (C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31)) {
-    // Tile choice.  Measured over M = 64 .. 8192 at the GPT-2 shapes, a launch takes
-    // about  fixed + ceil(tiles / 256 CUs) x (tile area x K) / (per-CU MFMA rate x eff)
-    // with eff = 1 / 0.985 / 0.89 / 0.77 for the four tile shapes (smaller tiles move
-    // more bytes into LDS per MFMA), so the tile with the least
-    // ceil(tiles / 256) x area / eff wins: 128x192 for large problems, 64x64 or 32x32
-    // for short prompts and small batches, where they still fill the chip.  The clock
-    // probe exists for the two large shapes only.
-    struct Cand { int bm, bn; double eff; };
-    const Cand cands[] = {{128, 192, 1.00}, {128, 128, 0.985}, {64, 64, 0.89}, {32, 32, 0.77}};
-    int best = 0;
-    double best_cost = 0;
-    long long best_tiles = 0;
-    for (int i = 0; i < (probe ? 2 : 4); i++) {
-      const long long t = (long long)((M + cands[i].bm - 1) / cands[i].bm) *
-                          ((OC + cands[i].bn - 1) / cands[i].bn);
-      const double cost = (double)((t + 255) / 256) * cands[i].bm * cands[i].bn / cands[i].eff;
-      if (i == 0 || cost < best_cost) {
-        best = i;
-        best_cost = cost;
-        best_tiles = t;
-      }
-    }
+    const TileChoice choice = choose_tile(M, C, OC, probe != nullptr);
+    const int best = choice.index;
+    const long long best_tiles = choice.tiles;
     if (best_tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
     if (probe_groups) *probe_groups = (int)best_tiles;
     switch (best) {
-      case 3:
+      case 5:
         // one 32x32 tile per workgroup, its four waves splitting K
         return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu);
-      case 2:
+      case 4:
         // up to two tiles per CU: latency-bound, ring of four slabs and a 2-way K split
         if (best_tiles <= 2 * 256)
           return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu);
         return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu);
+      case 3:
+        return launch_dma<64, 128, 2, 2>(out, inp, weight, bias, M, C, OC, gelu);
+      case 2:
+        // four waves of 32x96: two workgroups per compute unit
+        return launch_dma<128, 96, 4, 1>(out, inp, weight, bias, M, C, OC, gelu);
       case 1:
-        return launch_dma<128, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+        return launch_dma<128, 128, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
       default:
         // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
         // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
         // gives every SIMD two waves to alternate between.
         if (best_tiles >= 16 * 256)
-          return launch_dma<128, 192, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
-        return launch_dma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, probe);
+          return launch_dma<128, 192, 2, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
+        return launch_dma<128, 192, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
     }
   }
   if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs C %% 32 == 0");
@@ -1259,6 +1296,21 @@ int matmul_forward_probe_status(float* out, const float* inp, const float* weigh
     return fail(GPT2HIP_EINVAL, "matmul_forward_probe: probe buffer holds %d workgroups, need %lld",
                 probe_capacity, most);
   return matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false, probe, workgroups);
+}
+
+int matmul_forward_tile_shape(int B, int T, int C, int OC, int* tile_rows, int* tile_cols) {
+  using namespace g2;
+  const long long M64 = (long long)B * T;
+  if (B < 1 || T < 1 || C < 1 || OC < 1 || M64 > 0x7fffffffLL || !tile_rows || !tile_cols)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_tile_shape: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
+  if (C % BK != 0 || M64 <= 16 || (long long)C * 192 * 4 >= (1LL << 31)) {
+    *tile_rows = *tile_cols = 0;  // not one of the tiled LDS-DMA kernels
+    return GPT2HIP_OK;
+  }
+  const TileChoice c = choose_tile((int)M64, C, OC, false);
+  *tile_rows = c.bm;
+  *tile_cols = c.bn;
+  return GPT2HIP_OK;
 }
 
 size_t matmul_forward_argmax_workspace(int B, int T, int OC) {

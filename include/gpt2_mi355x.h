@@ -81,6 +81,14 @@ int matmul_forward_status(float* out, const float* inp, const float* weight, con
 void matmul_forward(float* out, const float* inp, const float* weight, const float* bias, int B,
                     int T, int C, int OC);
 
+/* Which workgroup tile (rows x columns of the product) matmul_forward gives a problem:
+ * 128x192, 128x128, 128x96, 64x128, 64x64 or 32x32, chosen by a fitted
+ * cost model so that the tiles come out in close to whole rounds over the 256 compute units
+ * (the reference launches one fixed 128x128 tile shape and asserts divisibility,
+ * kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:266-274).  Both are 0 for problems that
+ * take another kernel (C % 32 != 0, B*T <= 16).  Touches no GPU. */
+int matmul_forward_tile_shape(int B, int T, int C, int OC, int* tile_rows, int* tile_cols);
+
 /* Same with tanh-GELU applied to the result when is_gelu != 0.  Replaces
  * matmul_forward_async_cg_tf32_gelu, reference
  * kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:237-246. */

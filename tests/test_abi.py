@@ -78,3 +78,29 @@ def test_bench_refuses_more_than_one_gpu():
     proc = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=300)
     assert proc.returncode != 0
     assert "--gpus 1" in (proc.stdout + proc.stderr)
+
+
+def test_tile_choice_needs_no_gpu_and_avoids_partial_rounds():
+    """The GEMM's tile choice: 124M at B*T = 8192 keeps the largest tile (3, 1, 4, 1 whole
+    rounds of 256 tiles), the same layer shapes at B*T = 4096 take the tile that divides
+    evenly (128x96: 768 and 256 tiles instead of 384 and 128 tiles of 128x192)."""
+    import importlib
+    g2 = importlib.import_module("cuda-gpt2-inference_amd")
+    for C, OC in ((768, 2304), (768, 768), (768, 3072), (3072, 768)):
+        assert g2.matmul_forward_tile_shape(8, 1024, C, OC) == (128, 192)
+    assert g2.matmul_forward_tile_shape(4, 1024, 768, 2304) == (128, 96)
+    assert g2.matmul_forward_tile_shape(4, 1024, 768, 768) == (128, 96)
+    assert g2.matmul_forward_tile_shape(4, 1024, 1024, 1024) == (128, 128)      # 350M
+    assert g2.matmul_forward_tile_shape(8, 1024, 768, 50257) == (128, 192)      # lm-head
+    assert g2.matmul_forward_tile_shape(4, 64, 768, 768) == (32, 32)            # short prompt
+    assert g2.matmul_forward_tile_shape(1, 100, 36, 200) == (0, 0)              # K % 32 != 0
+    assert g2.matmul_forward_tile_shape(1, 16, 768, 768) == (0, 0)              # <= 16 rows
+    # whatever is chosen never needs more rounds of work than the largest tile would
+    for M in range(64, 8193, 448):
+        for C, OC in ((768, 2304), (768, 768), (1024, 4096), (4096, 1024)):
+            bm, bn = g2.matmul_forward_tile_shape(1, M, C, OC)
+            rounds = -(-(-(-M // bm) * -(-OC // bn)) // 256)
+            big = -(-(-(-M // 128) * -(-OC // 192)) // 256)
+            assert rounds * bm * bn <= big * 128 * 192 * 1.45, (M, C, OC, bm, bn)
+    with pytest.raises(g2.GPT2HipError):
+        g2.matmul_forward_tile_shape(0, 5, 32, 32)

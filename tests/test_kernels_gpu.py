@@ -227,6 +227,25 @@ def test_matmul_bias(M, C, OC):
     assert_close(out, oracle.matmul_forward(x, w, b), "matmul")
 
 
+# Problems whose tile count does not come out in whole rounds of 256 with the largest tile
+# (GPT-2 124M at B*T = 4096, 2048, 6144, ...), each with ragged edges in both dimensions, one
+# or more per tile shape of the dispatcher; the expected shape is asserted so that the list
+# keeps covering all of them.
+@pytest.mark.parametrize("M,C,OC,tile", [
+    (4096, 768, 2304, (128, 96)), (4093, 768, 2301, (128, 96)), (4096, 3072, 768, (128, 96)),
+    (2048, 768, 768, (64, 128)), (2045, 768, 771, (64, 128)), (6140, 768, 2300, (64, 128)),
+    (2048, 768, 2304, (64, 64)), (3070, 1024, 1000, (64, 64)),
+    (1536, 768, 2304, (128, 128)), (4090, 1024, 1020, (128, 128)),
+    (2048, 768, 3072, (128, 192)), (500, 768, 2304, (32, 32)),
+])
+def test_matmul_every_tile_shape_with_edges(M, C, OC, tile):
+    say(f"matmul M={M} C={C} OC={OC} tile={tile}")
+    assert g2.matmul_forward_tile_shape(1, M, C, OC) == tile
+    x, w, b = mm_inputs(M, C, OC, 123)
+    out = run_matmul(x, w, b)
+    assert_close(out, oracle.matmul_forward(x, w, b), "matmul")
+
+
 def test_matmul_lm_head_no_bias():
     # 768 -> 50257 without bias; the oracle runs on a row subset to stay in seconds,
     # which is exact because rows are independent.
