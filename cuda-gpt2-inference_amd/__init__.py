@@ -49,7 +49,7 @@ EXPORTS = (
     "gpt2_create", "gpt2_destroy", "gpt2_num_parameters", "gpt2_params_device",
     "gpt2_load_params_host", "gpt2_reserve", "gpt2_forward", "gpt2_forward_status",
     "gpt2_forward_device_status", "gpt2_forward_graph_status",
-    "gpt2_prefill_status", "gpt2_decode_status", "gpt2_decode_options", "gpt2_decode_probe_status", "gpt2_decode_probe_size",
+    "gpt2_prefill_status", "gpt2_decode_status", "gpt2_decode_sync_status", "gpt2_decode_options", "gpt2_decode_probe_status", "gpt2_decode_probe_size",
     "gpt2_step_logits", "gpt2_cache_length",
     "gpt2_forward_argmax_status",
     "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
@@ -153,6 +153,7 @@ def lib() -> ctypes.CDLL:
         L.gpt2_prefill_status.argtypes, L.gpt2_prefill_status.restype = [vp, vp, ci, ci], ci
         L.gpt2_decode_status.argtypes, L.gpt2_decode_status.restype = [vp, vp], ci
         L.gpt2_decode_options.argtypes, L.gpt2_decode_options.restype = [vp, ci, ctypes.c_uint], ci
+        L.gpt2_decode_sync_status.argtypes, L.gpt2_decode_sync_status.restype = [vp], ci
         L.gpt2_decode_probe_status.argtypes, L.gpt2_decode_probe_status.restype = [vp, vp, vp, cz], ci
         L.gpt2_decode_probe_size.argtypes, L.gpt2_decode_probe_size.restype = [vp], cz
         L.gpt2_step_logits.argtypes, L.gpt2_step_logits.restype = [vp], vp
@@ -426,7 +427,13 @@ class GPT2:
             argmax_forward(out[s], logits, B, V)
             if s + 1 < steps:
                 logits = self.decode(out[s])
+        self.decode_sync()  # a step that failed on the device would have left NaN logits behind
         return out.t().contiguous()
+
+    def decode_sync(self) -> None:
+        """Wait for the decode steps queued so far; raises if one of them gave up on the device
+        (the cache is then rolled back to the positions before it, see cache_length())."""
+        _check(lib().gpt2_decode_sync_status(self._h), "gpt2_decode_sync")
 
     def decode_probe(self, next_ids_device):
         """One decode step of the persistent kernel with its clock probe: returns a

@@ -33,9 +33,9 @@
 // of per-workgroup epoch flags accessed the same way: a workgroup waits for its own
 // stores to be acknowledged, publishes the phase number, and polls everybody's flag.
 // Weights and the cache rows of earlier steps are read-only for the kernel and go through
-// the caches normally.  Every wait is bounded: a workgroup that spins too long raises an
-// error word that makes every workgroup leave the kernel, and the host reports it on a
-// later call.
+// the caches normally.  Every wait is bounded: a workgroup that spins too long writes the
+// step's position into an error word that makes every workgroup leave the kernel -- each
+// filling the logits it owns with NaN -- and the host reports it when it next looks.
 #include "common.hpp"
 
 namespace g2 {
@@ -145,9 +145,10 @@ __device__ __forceinline__ bool grid_wait(const DecodeStep& a, float* lds, unsig
       if (all) break;
       __builtin_amdgcn_s_sleep(2);
       ++spins;
-      if (spins > a.spin_limit ||
-          ((spins & 63) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-        __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool seen = (spins & 63) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (spins > a.spin_limit || seen) {
+        // the error word names the step that failed first: position + 1, written once
+        if (!seen) atomicCAS(err, 0u, (unsigned)a.pos + 1u);
         *bad = 1;
         break;
       }
@@ -678,6 +679,20 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   }
 }
 
+// A step that ends early must not leave the previous step's logits behind as if they were its
+// own: every workgroup that leaves fills the logits it owns in the lm-head phase (the same
+// 16-row groups, for every sequence) with NaN.  Nobody else writes those, so they stay NaN
+// whatever the other workgroups still manage to do.
+__device__ __forceinline__ void fail_logits(const DecodeStep& a) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int step = (int)gridDim.x * DS_WAVES;
+  for (int cg = lm_head_first_group(wave); cg * 16 < a.V; cg += step) {
+    const int n = cg * 16 + (lane & 15);
+    if (n < a.V)
+      for (int b = lane >> 4; b < a.B; b += 4) a.logits[(size_t)b * a.V + n] = __builtin_nanf("");
+  }
+}
+
 // KG1 = C / 256: groups of 64 k per wave where K = C, and weight rows per workgroup where
 // N = C (the grid is exactly DS_GRID = 256 workgroups).  JG: groups of 4 sequences.
 // ULM: units of 16 k per chunk of the lm-head's sweep.
@@ -687,12 +702,15 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
   constexpr int C = 256 * KG1;
   constexpr size_t cs = (size_t)C;
   unsigned* const err = a.flags + (size_t)gridDim.x * FLAG_STRIDE;
-  // a launch that follows a failed one does nothing until the host has cleared the error
+  // a launch that follows a failed one computes nothing until the host has cleared the error
   if (threadIdx.x == 0)
     *reinterpret_cast<int*>(lds + LDS_BAD) =
         __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
   __syncthreads();
-  if (*reinterpret_cast<int*>(lds + LDS_BAD) != 0) return;
+  if (*reinterpret_cast<int*>(lds + LDS_BAD) != 0) {
+    fail_logits(a);
+    return;
+  }
   unsigned epoch = a.epoch0;
 
   const int items = a.B * a.NH * a.att_splits;  // (sequence, head, range) triples of the attention phase
@@ -712,7 +730,10 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
     else
       gemm_phase<true, false, false, true, false>(a, lds, w_qkv, a.x, a.qkv, nullptr, next_proj);
     grid_arrive(a, ++epoch);
-    if (!grid_wait(a, lds, epoch)) return;
+    if (!grid_wait(a, lds, epoch)) {
+      fail_logits(a);
+      return;
+    }
 
     // attention over the cache
     // at most one item per workgroup: B <= 16 sequences of at most 1024 / 64 heads, and the
@@ -722,21 +743,30 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
       attention_item(a, lds, kc, vc, bh / a.NH, bh % a.NH, (int)blockIdx.x % a.att_splits);
     }
     grid_arrive(a, ++epoch);
-    if (!grid_wait(a, lds, epoch)) return;
+    if (!grid_wait(a, lds, epoch)) {
+      fail_logits(a);
+      return;
+    }
 
     // x += y Wproj + b
     gemm_phase<false, false, false, false, true>(a, lds, w_proj, a.atty, a.x, a.x, [&]() {
       load_phase_weights(w_fc, a.fcw + l * 4 * cs * cs, a.fcb + l * 4 * cs, a.ln2w + l * cs, a.ln2b + l * cs);
     });
     grid_arrive(a, ++epoch);
-    if (!grid_wait(a, lds, epoch)) return;
+    if (!grid_wait(a, lds, epoch)) {
+      fail_logits(a);
+      return;
+    }
 
     // h = gelu(LN2(x) Wfc + b)
     gemm_phase<true, true, false, false, false>(a, lds, w_fc, a.x, a.h, nullptr, [&]() {
       load_phase_weights(w_fcproj, a.fcprojw + l * 4 * cs * cs, a.fcprojb + l * cs, nullptr, nullptr);
     });
     grid_arrive(a, ++epoch);
-    if (!grid_wait(a, lds, epoch)) return;
+    if (!grid_wait(a, lds, epoch)) {
+      fail_logits(a);
+      return;
+    }
 
     // x += h Wfcproj + b
     gemm_phase<false, false, false, false, false>(a, lds, w_fcproj, a.h, a.x, a.x, [&]() {
@@ -745,7 +775,10 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
                            a.ln1w + (l + 1) * cs, a.ln1b + (l + 1) * cs);
     });
     grid_arrive(a, ++epoch);
-    if (!grid_wait(a, lds, epoch)) return;
+    if (!grid_wait(a, lds, epoch)) {
+      fail_logits(a);
+      return;
+    }
   }
   lm_head_phase<4 * KG1, ULM>(a, lds);
   trace_mark(a, 5u * (unsigned)a.L, 0);
@@ -754,14 +787,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
 // ---- host ---------------------------------------------------------------------------------
 // The kernel runs on exactly DS_GRID workgroups, one per compute unit, all resident at once.
 static bool device_has_grid(int device) {
-  static int cached_device = -1, cached = 0;
-  if (device != cached_device) {
-    int cus = 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return false;
-    cached_device = device;
-    cached = cus;
-  }
-  return cached >= DS_GRID;
+  int cus = 0;  // a cached attribute of the runtime: no state of our own to keep per device or thread
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return false;
+  return cus >= DS_GRID;
 }
 
 size_t decode_step_flag_bytes(int device) {
@@ -830,10 +858,20 @@ int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) 
                        : kg1 == 2 ? kernel_for<2, 16>(jg)
                        : kg1 == 3 ? kernel_for<3, 24>(jg)
                                   : kernel_for<4, 16>(jg);
-  static bool lds_raised[4][4] = {};
-  if (lds > 48 * 1024 && !lds_raised[kg1 - 1][jg - 1]) {
-    G2_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    lds_raised[kg1 - 1][jg - 1] = true;
+  // the dynamic-LDS limit is a per-device property of the kernel: remembered per thread and
+  // device, like the GEMM launchers do
+  if (lds > 48 * 1024) {
+    static thread_local int raised_on = -1;
+    static thread_local bool raised[4][4];
+    if (raised_on != device) {
+      raised_on = device;
+      for (auto& row : raised)
+        for (bool& b : row) b = false;
+    }
+    if (!raised[kg1 - 1][jg - 1]) {
+      G2_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+      raised[kg1 - 1][jg - 1] = true;
+    }
   }
   // An ordinary launch: with one workgroup per compute unit's worth of resources and nothing
   // else running on the device, all DS_GRID workgroups are resident at once, which the grid

@@ -68,6 +68,9 @@ struct GPT2 {
   float* step_act;  // the activations it hands between workgroups (decode_step_activation_floats)
   unsigned step_epoch;
   unsigned* step_error_host;
+  hipEvent_t step_event;     // recorded behind every copy of the error word to step_error_host
+  bool step_pending;         // a step has been launched whose copy has not been looked at yet
+  bool step_fallback;        // a step of the persistent kernel gave up: one launch per operation from then on
   bool step_persistent;      // use the persistent kernel where it takes the model
   unsigned step_spin_limit;  // polls of a barrier flag before a workgroup gives up
 
@@ -111,6 +114,9 @@ static void free_cache(GPT2* m) {
   if (m->step_act) (void)hipFree(m->step_act);
   m->step_act = nullptr;
   if (m->step_error_host) (void)hipHostFree(m->step_error_host);
+  if (m->step_event) (void)hipEventDestroy(m->step_event);
+  m->step_event = nullptr;
+  m->step_pending = false;
   m->kv = m->step_logits = nullptr;
   m->step_flags = m->step_error_host = nullptr;
   m->step_epoch = 0;
@@ -134,6 +140,7 @@ static int reserve_cache(GPT2* m, int B) {
   if (e == hipSuccess) e = hipMemset(m->step_act, 0, act_bytes);
   if (e == hipSuccess) e = hipHostMalloc((void**)&m->step_error_host, sizeof(unsigned), hipHostMallocDefault);
   if (e == hipSuccess) *m->step_error_host = 0;
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&m->step_event, hipEventDisableTiming);
   if (e != hipSuccess) {
     free_cache(m);
     return fail(GPT2HIP_ENOMEM, "gpt2: key/value cache for %d sequences (%zu bytes): %s", B, kv_bytes,
@@ -512,8 +519,49 @@ int gpt2_forward_graph_status(GPT2* model, const int* inputs_device, int B, int 
   return GPT2HIP_OK;
 }
 
+namespace g2 {
+// Looks at the error word of the persistent decode-step kernel once the copy behind the
+// newest step has arrived (wait: block until it has; otherwise only if it already has).  A
+// step that gave up a barrier wait left NaN logits, and so did every step queued behind it;
+// the word names its position.  Recovery: the cache is rolled back to the positions before
+// that step, the barrier state is cleared, and the model decodes with one launch per
+// operation from then on.  Returns an error exactly once per failure.
+static int settle_steps(GPT2* m, bool wait) {
+  if (!m->step_pending) return GPT2HIP_OK;
+  if (wait) {
+    G2_HIP(hipEventSynchronize(m->step_event));
+  } else {
+    const hipError_t q = hipEventQuery(m->step_event);
+    if (q == hipErrorNotReady) return GPT2HIP_OK;
+    G2_HIP(q);
+  }
+  m->step_pending = false;
+  const unsigned word = *m->step_error_host;
+  if (word == 0) return GPT2HIP_OK;
+  *m->step_error_host = 0;
+  G2_HIP(hipMemsetAsync(m->step_flags, 0, decode_step_flag_bytes(m->device), stream()));
+  m->step_epoch = 0;
+  m->step_fallback = true;
+  const int failed = (int)word - 1;
+  if (m->kv_len > failed) m->kv_len = failed;
+  return fail(GPT2HIP_EHIP,
+              "gpt2_decode: the step at position %d gave up waiting at a grid barrier; its logits and "
+              "those of the steps queued behind it are NaN, the cache is rolled back to %d positions "
+              "and further steps run one launch per operation", failed, m->kv_len);
+}
+}  // namespace g2
+
+int gpt2_decode_sync_status(GPT2* model) {
+  if (!model) return g2::fail(GPT2HIP_EINVAL, "gpt2_decode_sync: null model");
+  return g2::settle_steps(model, true);
+}
+
 int gpt2_prefill_status(GPT2* model, const int* inputs_device, int B, int T) {
   using namespace g2;
+  if (!model) return fail(GPT2HIP_EINVAL, "gpt2_prefill: null model");
+  // a failure among earlier decode steps that nobody has asked about: the cache is rebuilt
+  // here anyway, so only the recovery (cleared barrier state, launch-per-operation steps) matters
+  (void)settle_steps(model, true);
   if (int rc = reserve(model, B, T)) return rc;
   if (!inputs_device) return fail(GPT2HIP_EINVAL, "gpt2_prefill: null inputs");
   if (model->kv_batch != B) {  // the cache planes are indexed with the batch it was sized for
@@ -550,7 +598,7 @@ int gpt2_decode_probe_status(GPT2* model, const int* next_ids_device, unsigned l
 
 size_t gpt2_decode_probe_size(const GPT2* model) {
   using namespace g2;
-  if (!model || !model->step_persistent || model->kv_batch < 1 ||
+  if (!model || !model->step_persistent || model->step_fallback || model->kv_batch < 1 ||
       !decode_step_supported(model->cfg, model->kv_batch, model->device))
     return 0;
   return decode_step_probe_slots(model->cfg.num_layers);
@@ -561,6 +609,9 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
   if (!model || !next_ids_device) return fail(GPT2HIP_EINVAL, "gpt2_decode: null pointer");
   GPT2* m = model;
   const GPT2Config& c = m->cfg;
+  // what is already known about earlier steps (never waits: steps are queued without
+  // synchronisation; a failure not yet visible here turns this step's logits into NaN too)
+  if (int rc = settle_steps(m, false)) return rc;
   if (m->kv_len < 1) return fail(GPT2HIP_EINVAL, "gpt2_decode: no prompt has been prefilled");
   if (m->kv_len >= c.max_seq_len)
     return fail(GPT2HIP_EINVAL, "gpt2_decode: the cache is full (%d positions)", c.max_seq_len);
@@ -578,20 +629,11 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
   float* other = m->res_b;
   G2_HIP(hipMemcpyAsync(m->ids, next_ids_device, (size_t)B * sizeof(int), hipMemcpyDeviceToDevice,
                         stream()));
-  const bool persistent = m->step_persistent && m->step_flags && m->step_act && decode_step_supported(c, B, m->device);
+  const bool persistent = m->step_persistent && !m->step_fallback && m->step_flags && m->step_act &&
+                          decode_step_supported(c, B, m->device);
   if (!persistent)  // the persistent kernel gathers the embeddings itself
     G2_TRY(encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
   const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
-  if (m->step_error_host && *m->step_error_host != 0) {
-    // an earlier step's kernel gave up a barrier wait: its logits and the cache row it was to
-    // append are not valid.  Clear the error so that a new prompt can run.
-    *m->step_error_host = 0;
-    G2_HIP(hipMemsetAsync(m->step_flags, 0, decode_step_flag_bytes(m->device), stream()));
-    m->step_epoch = 0;
-    m->kv_len = 0;
-    return fail(GPT2HIP_EHIP, "gpt2_decode: a workgroup of an earlier step gave up waiting at a grid "
-                              "barrier; the cache is invalid, prefill again");
-  }
   if (persistent) {
     // one persistent kernel for the whole step
     DecodeStep st;
@@ -638,6 +680,8 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
     G2_HIP(hipMemcpyAsync(m->step_error_host, (const char*)m->step_flags + decode_step_flag_bytes(m->device) -
                                                   16 * sizeof(unsigned),
                           sizeof(unsigned), hipMemcpyDeviceToHost, stream()));
+    G2_HIP(hipEventRecord(m->step_event, stream()));
+    m->step_pending = true;
   } else if (skinny_supported(B, C, true, residual, m->params) && skinny_supported(B, 4 * C, false, m->fch, m->params)) {
     // Up to 16 sequences: five launches per block.  The layernorms run inside the GEMMs
     // that consume them and the residual adds inside the GEMMs that produce the update:
@@ -689,6 +733,7 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
 
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit) {
   if (!model) return g2::fail(GPT2HIP_EINVAL, "gpt2_decode_options: null model");
+  if (persistent != 0) model->step_fallback = false;  // asked for (again) explicitly
   model->step_persistent = persistent != 0;
   model->step_spin_limit = spin_limit;
   return GPT2HIP_OK;

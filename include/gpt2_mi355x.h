@@ -228,9 +228,20 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device);
  * channels 256, 512, 768 or 1024, a device with at least 256 compute units), otherwise one
  * launch per operation; 0: always one launch per operation.  spin_limit bounds the polls a
  * workgroup of the persistent kernel spends on one flag of its grid barrier before it gives
- * up and ends the kernel (default 2^21); a step that gave up makes the NEXT gpt2_decode call
- * fail and empties the cache. */
+ * up and ends the kernel (default 2^21).  A step that gave up leaves NaN in gpt2_step_logits(),
+ * and so does every step already queued behind it (never stale values of an earlier step).
+ * The failure is reported once, by the first of gpt2_decode_status (if the step has ended by
+ * then: it never waits) or gpt2_decode_sync_status (which waits); by then the cache has been
+ * rolled back to the positions before the failed step (gpt2_cache_length()), so decoding can
+ * resume from there, and the model runs one launch per operation until gpt2_decode_options
+ * asks for the persistent kernel again.  gpt2_prefill_status clears a failure nobody asked
+ * about (it rebuilds the cache anyway). */
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit);
+/* Waits until every decode step queued so far has ended and reports whether one of the
+ * persistent kernel's steps gave up (see gpt2_decode_options); 0 if all of them completed.
+ * Call it before trusting ids or logits produced by steps that were queued without
+ * synchronisation.  No counterpart in the reference. */
+int gpt2_decode_sync_status(GPT2* model);
 /* One gpt2_decode step of the persistent kernel with a clock probe: every workgroup g records
  * the 100 MHz wall clock when it has finished the work of phase p (clocks[(2p) * G + g]) and
  * when it has passed the grid barrier after it (clocks[(2p + 1) * G + g]); phases are, per

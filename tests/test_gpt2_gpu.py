@@ -355,30 +355,61 @@ def test_gpt2_greedy_generation_equals_greedy_decoding_by_full_forward_passes(pe
 
 def test_gpt2_persistent_decode_gives_up_a_barrier_wait_cleanly():
     """Failure handling of the persistent kernel's grid barrier, forced from the host: with a
-    spin limit of 0 the first workgroup that has to wait gives up, every workgroup leaves the
-    kernel, a later call reports it, and the model works again after a new prompt."""
+    spin limit of 0 the first workgroup that has to wait gives up and every workgroup leaves the
+    kernel.  Steps are queued WITHOUT synchronisation, as generate_greedy queues them: none of
+    them may pass stale logits off as its own (they are NaN), the failure is reported by the
+    first call that can know of it, the cache is rolled back to the failed position, and the
+    model carries on from there with one launch per operation."""
     cfg = dict(max_seq_len=32, vocab_size=211, num_layers=2, num_heads=4, channels=256)
     params = syn.make_params(93, perturb_affine=True, **cfg)
-    ids = torch.from_numpy(syn.make_tokens(94, 2, 8, cfg["vocab_size"])).cuda()
+    ids = torch.from_numpy(syn.make_tokens(94, 2, 12, cfg["vocab_size"])).cuda()
     model = g2.GPT2(**cfg)
     try:
         model.load_params(params)
         model.decode_options(persistent=False)
         model.prefill(ids[:, :7].contiguous())
-        want = model.decode(ids[:, 7].contiguous()).clone()
+        want7 = model.decode(ids[:, 7].contiguous()).clone()
+        want8 = model.decode(ids[:, 8].contiguous()).clone()
         model.decode_options(persistent=True, spin_limit=0)
-        model.prefill(ids[:, :7].contiguous())
-        print("  step with spin limit 0", flush=True)
-        model.decode(ids[:, 7].contiguous())       # launches; some workgroup gives up
-        torch.cuda.synchronize()                   # the kernel has ended by itself
-        with pytest.raises(g2.GPT2HipError, match="grid barrier"):
-            model.decode(ids[:, 7].contiguous())
-        assert model.cache_length() == 0
+        stale = model.prefill(ids[:, :7].contiguous()).clone()   # finite logits of position 6
+        print("  three steps with spin limit 0, queued without synchronisation", flush=True)
+        seen = []
+        try:
+            for t in (7, 8, 9):                                   # the first one gives up on the device
+                seen.append(model.decode(ids[:, t].contiguous()).clone())
+        except g2.GPT2HipError as e:                              # allowed: the host already knew
+            assert "grid barrier" in str(e)
+        with_error = False
+        try:
+            model.decode_sync()
+        except g2.GPT2HipError as e:
+            assert "grid barrier" in str(e) and "position 7" in str(e)
+            with_error = True
+        torch.cuda.synchronize()
+        assert with_error or len(seen) < 3, "the failure was never reported"
+        for lg in seen:                                           # never finite stale values
+            assert torch.isnan(lg).any() and not torch.equal(lg, stale)
+        assert model.cache_length() == 7                          # rolled back to the failed step
+        print("  resumed from the rolled-back cache, one launch per operation", flush=True)
+        got7 = model.decode(ids[:, 7].contiguous()).clone()
+        got8 = model.decode(ids[:, 8].contiguous()).clone()
+        model.decode_sync()
+        assert (got7 - want7).abs().max().item() <= 1e-4
+        assert (got8 - want8).abs().max().item() <= 1e-4
+        # asking for the persistent kernel again brings it back, after a new prompt or not
         model.decode_options(persistent=True)
         model.prefill(ids[:, :7].contiguous())
         got = model.decode(ids[:, 7].contiguous())
-        torch.cuda.synchronize()
-        assert (got - want).abs().max().item() <= 1e-4
+        model.decode_sync()
+        assert (got - want7).abs().max().item() <= 1e-4
+        # a failure nobody asked about does not outlive the next prompt
+        model.decode_options(persistent=True, spin_limit=0)
+        model.decode(ids[:, 8].contiguous())
+        model.decode_options(persistent=True)
+        model.prefill(ids[:, :7].contiguous())
+        got = model.decode(ids[:, 7].contiguous())
+        model.decode_sync()
+        assert (got - want7).abs().max().item() <= 1e-4
     finally:
         model.close()
 
