@@ -105,6 +105,19 @@ def time_launch(g2, fn, iters=30, warmup=10, groups=5):
     return sorted(per_launch)[len(per_launch) // 2]
 
 
+def marker_overhead_ms(g2):
+    """What one event between two launches adds to the interval it closes.  The profiled
+    forward records an event after every launch and charges a launch the time between its two
+    events: the launch-to-launch time PLUS the event marker's own trip through the command
+    processor.  The library measures it the way it records those events, on launches that do
+    next to nothing (median of five runs of 64 launches)."""
+    L = g2.lib()
+    us = sorted(L.gpt2hip_profile_marker_overhead_us(64) for _ in range(5))
+    if us[0] < 0:
+        raise RuntimeError("gpt2hip_profile_marker_overhead_us failed")
+    return us[2] / 1e3
+
+
 def standalone(g2):
     """Per-kernel figures at the BASELINE shapes (configs 1-3).
 
@@ -466,17 +479,24 @@ def main():
     flops = forward_flops(cfg, B, T)
     nbytes = forward_bytes(cfg, B, T)
     L = cfg["num_layers"]
+    marker_ms = marker_overhead_ms(g2)
+    log(f"  event marker between two launches: +{marker_ms * 1e3:.2f} us per interval")
     kernels = []
     for k in g2.PROF_CATEGORIES:
         launches = LAUNCHES.get(k, 2 * L if k == "fused_residual_layernorm" else L)
         row = {"launch": k, "launches_per_forward": launches, "ms_per_forward": prof[k],
                "ms_per_launch": prof[k] / launches}
+        # the same figure with the event marker's own cost taken out of every interval: what a
+        # launch takes from the end of its predecessor to its own end, as in an unprofiled pass
+        net = max(prof[k] - launches * marker_ms, 1e-9)
         if k in flops:
             tf = flops[k] / prof[k] / 1e9
-            row.update({"TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS})
+            row.update({"TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS,
+                        "frac_fp32_mfma_net_of_marker": flops[k] / net / 1e9 / PEAK_FP32_MFMA_TFLOPS})
         else:
             gbs = nbytes[k] / prof[k] / 1e6
             row.update({"GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
+                        "frac_hbm_net_of_marker": nbytes[k] / net / 1e6 / PEAK_HBM_GBS,
                         "note": "inside the forward pass, operands may be served by the 256 MiB "
                                 "Infinity Cache"})
         kernels.append(row)
@@ -494,6 +514,8 @@ def main():
                 "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                 "traffic": (DOMINANT_TRAFFIC_BYTES
                             if (args.model == "124M" and B == 8 and T == 1024) else None),
+                "traffic_source": "recorded from two rocprofv3 --pmc runs of bench.py --pmc-probe "
+                                  "(profiles/kernels_baseline_shapes_pmc.txt), not counted in this run",
                 "kernel": ("matmul_dma_kernel<128,192,4,2,false>" if B * T == 8192 else
                            "matmul_forward, qkv / attproj / fcproj launches (tile shape by size)"),
                 "avg_launch_ms": dom_ms, "flops_per_launch": dom_flops,
@@ -512,6 +534,10 @@ def main():
         "kernels": kernels,
     }
     result["host_ids_ms_per_step"] = host_ids_ms
+    result["profile_marker_overhead_us"] = marker_ms * 1e3
+    result["profile_note"] = ("kernels[].ms_per_launch is the time between the events recorded before "
+                              "and after a launch, which includes the closing event's own "
+                              "profile_marker_overhead_us; the *_net_of_marker fractions take that out")
     if graph_ms is not None:
         result["graph_replay_ms_per_step"] = graph_ms
     if not args.no_standalone:

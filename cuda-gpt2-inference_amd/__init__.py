@@ -52,7 +52,7 @@ EXPORTS = (
     "gpt2_prefill_status", "gpt2_decode_status", "gpt2_decode_sync_status", "gpt2_decode_options", "gpt2_decode_probe_status", "gpt2_decode_probe_size",
     "gpt2_step_logits", "gpt2_cache_length",
     "gpt2_forward_argmax_status",
-    "gpt2_forward_profiled_status", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
+    "gpt2_forward_profiled_status", "gpt2hip_profile_marker_overhead_us", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
     "gpt2hip_timer_stop_ms",
 )
@@ -172,6 +172,8 @@ def lib() -> ctypes.CDLL:
         L.matmul_forward_argmax_noalloc_status.restype = ci
         L.gpt2_forward_profiled_status.argtypes = [vp, vp, ci, ci, ctypes.POINTER(ctypes.c_float)]
         L.gpt2_forward_profiled_status.restype = ci
+        L.gpt2hip_profile_marker_overhead_us.argtypes = [ci]
+        L.gpt2hip_profile_marker_overhead_us.restype = ctypes.c_float
         L.gpt2_logits.argtypes, L.gpt2_logits.restype = [vp], vp
         L.gpt2_lnf.argtypes, L.gpt2_lnf.restype = [vp], vp
         L.gpt2_argmax_status.argtypes, L.gpt2_argmax_status.restype = [vp, vp], ci
@@ -342,8 +344,8 @@ class Timer:
         return float(ms)
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            lib().gpt2hip_timer_destroy(self._h)
+        if getattr(self, "_h", None) and _lib is not None:  # at interpreter exit the module may be gone
+            _lib.gpt2hip_timer_destroy(self._h)
             self._h = None
 
 

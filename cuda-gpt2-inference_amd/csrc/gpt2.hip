@@ -12,6 +12,8 @@
 #include <cstring>
 #include <vector>
 
+#include <dlfcn.h>
+
 #include "common.hpp"
 
 namespace g2 {
@@ -188,6 +190,33 @@ static int reserve(GPT2* m, int B, int T) {
 // Optional per-launch timing: an event is recorded on the null stream before the
 // first launch and after every launch; category[i] names the launch between
 // events i and i+1.
+// Named ranges around the launches of the profiled forward pass, for a rocprofv3 marker
+// trace (the counterpart of the reference's NVTX ranges, kernels/attention/
+// 1_attention_cublas.cuh:44-67).  The marker library is looked up at run time, once: without
+// it (or outside a profiler) the ranges are no-ops, and the timed entry points never touch it.
+struct Roctx {
+  int (*push)(const char*) = nullptr;
+  int (*pop)() = nullptr;
+  Roctx() {
+    void* h = dlopen("librocprofiler-sdk-roctx.so", RTLD_NOW | RTLD_LOCAL);
+    if (!h) h = dlopen("librocprofiler-sdk-roctx.so.1", RTLD_NOW | RTLD_LOCAL);
+    if (!h) return;
+    push = reinterpret_cast<int (*)(const char*)>(dlsym(h, "roctxRangePushA"));
+    pop = reinterpret_cast<int (*)()>(dlsym(h, "roctxRangePop"));
+    if (!push || !pop) push = nullptr, pop = nullptr;
+  }
+};
+static const Roctx& roctx() {
+  static const Roctx r;  // thread-safe initialisation
+  return r;
+}
+static const char* const kProfNames[GPT2_PROF_COUNT] = {
+    "encoder_forward",       "layernorm_forward",
+    "matmul_forward qkv",    "attention_forward",
+    "matmul_forward attproj", "fused_residual_layernorm_forward",
+    "matmul_forward_gelu fc", "matmul_forward fcproj",
+    "matmul_forward lm-head"};
+
 struct Profile {
   std::vector<hipEvent_t> events;
   std::vector<int> category;
@@ -219,10 +248,13 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
   do {                                \
     if (int rc_ = (call)) return rc_; \
   } while (0)
-#define G2_STEP(cat, call)                \
-  do {                                    \
-    G2_TRY(call);                         \
-    if (prof) G2_TRY(prof->mark(cat));    \
+#define G2_STEP(cat, call)                                   \
+  do {                                                       \
+    if (prof && roctx().push) roctx().push(kProfNames[cat]); \
+    const int rc_step_ = (call);                             \
+    if (prof && roctx().pop) roctx().pop();                  \
+    if (rc_step_) return rc_step_;                           \
+    if (prof) G2_TRY(prof->mark(cat));                       \
   } while (0)
   if (prof) G2_TRY(prof->mark(-1));
 
@@ -771,6 +803,42 @@ int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, i
     ms_per_category[prof.category[i]] += ms;
   }
   return GPT2HIP_OK;
+}
+
+float gpt2hip_profile_marker_overhead_us(int launches) {
+  using namespace g2;
+  if (launches < 1) launches = 64;
+  float* buf = nullptr;
+  if (hipMalloc((void**)&buf, 256 * sizeof(float)) != hipSuccess) {
+    fail(GPT2HIP_ENOMEM, "gpt2hip_profile_marker_overhead_us: hipMalloc failed");
+    return -1.f;
+  }
+  float result = -1.f;
+  do {
+    if (hipMemsetAsync(buf, 0, 256 * sizeof(float), stream()) != hipSuccess) break;
+    for (int i = 0; i < launches; i++)
+      if (residual_forward_status(buf, buf, buf, 256)) break;
+    // (a) an event after every launch, as gpt2_forward_profiled_status records them
+    Profile prof;
+    if (prof.mark(-1)) break;
+    bool ok = true;
+    for (int i = 0; i < launches && ok; i++) ok = !residual_forward_status(buf, buf, buf, 256) && !prof.mark(0);
+    if (!ok || hipEventSynchronize(prof.events.back()) != hipSuccess) break;
+    float marked = 0.f;
+    if (hipEventElapsedTime(&marked, prof.events.front(), prof.events.back()) != hipSuccess) break;
+    // (b) the same launches back to back between two events
+    Profile bare;
+    if (bare.mark(-1)) break;
+    for (int i = 0; i < launches && ok; i++) ok = !residual_forward_status(buf, buf, buf, 256);
+    if (!ok || bare.mark(0) || hipEventSynchronize(bare.events.back()) != hipSuccess) break;
+    float plain = 0.f;
+    if (hipEventElapsedTime(&plain, bare.events.front(), bare.events.back()) != hipSuccess) break;
+    result = (marked - plain) * 1000.f / (float)launches;
+    if (result < 0.f) result = 0.f;
+  } while (false);
+  (void)hipFree(buf);
+  if (result < 0.f) fail(GPT2HIP_EHIP, "gpt2hip_profile_marker_overhead_us: a HIP call failed");
+  return result;
 }
 
 const float* gpt2_logits(const GPT2* model) { return model ? model->logits : nullptr; }

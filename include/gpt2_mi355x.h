@@ -128,8 +128,13 @@ void argmax_forward(int* ids, const float* logits, int N, int V);
 /* matmul_forward followed by argmax_forward without the (B*T, OC) product ever reaching
  * memory: ids[r] = argmax_o (inp[r,:] . weight[o,:] + bias[o]), lowest index wins ties.
  * For C % 32 == 0 and 16-byte aligned operands (the lm-head) the GEMM's tiles are reduced
- * to (value, column) pairs in their epilogue and a second small kernel reduces the pairs;
- * the result equals argmax_forward over matmul_forward's output exactly.  workspace is
+ * to (value, column) pairs in their epilogue and a second small kernel reduces the pairs.
+ * The products are accumulated over C in ascending order, as every tiled kernel of
+ * matmul_forward accumulates them, so wherever matmul_forward does not split C between
+ * waves the ids equal argmax_forward over matmul_forward's output bit for bit (it splits C
+ * for B*T <= 16, for 32x32 tiles and for up to 512 tiles of 64x64: small problems; a GPT-2
+ * lm-head of 64 or more rows is not among them).  Where it does, the two can differ where
+ * logits tie to within rounding.  workspace is
  * device memory of at least matmul_forward_argmax_workspace(B, T, OC) bytes.  Other shapes
  * take a slow one-block-per-row kernel and ignore the workspace.  No counterpart in the
  * reference, which runs its matmul launcher (kernels/matmul/2_matmul_cublas.cuh:34) and
@@ -277,6 +282,12 @@ enum {
 };
 int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, int T,
                                  float* ms_per_category);
+/* What the event that gpt2_forward_profiled_status records after a launch adds to the
+ * interval it closes, in microseconds: `launches` launches that do next to nothing, timed with
+ * an event after each one and again back to back, difference per launch.  Allocates and frees
+ * 1 KiB of device memory and waits for its launches; negative on failure.  For reading the
+ * per-category times of short kernels (a diagnostic, like the profiled pass itself). */
+float gpt2hip_profile_marker_overhead_us(int launches);
 const float* gpt2_logits(const GPT2* model);
 /* Final layernorm output (B,T,C) of the last forward, on the device. */
 const float* gpt2_lnf(const GPT2* model);
