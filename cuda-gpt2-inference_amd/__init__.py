@@ -41,6 +41,8 @@ EXPORTS = (
     "matmul_forward", "matmul_forward_status",
     "matmul_forward_gelu", "matmul_forward_gelu_status", "matmul_forward_probe_status",
     "matmul_forward_tile_shape",
+    "matmul_forward_splitk_workspace", "matmul_forward_splitk_status",
+    "matmul_forward_splitk_plan", "matmul_forward_splitk_forced_status",
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
     "matmul_forward_argmax_workspace", "matmul_forward_argmax_status",
@@ -136,6 +138,14 @@ def lib() -> ctypes.CDLL:
         L.matmul_forward_probe_status.restype = ci
         L.matmul_forward_tile_shape.argtypes = [ci] * 4 + [ctypes.POINTER(ci)] * 2
         L.matmul_forward_tile_shape.restype = ci
+        L.matmul_forward_splitk_workspace.argtypes = []
+        L.matmul_forward_splitk_workspace.restype = cz
+        L.matmul_forward_splitk_status.argtypes = [vp] * 4 + [ci] * 5 + [vp, cz]
+        L.matmul_forward_splitk_status.restype = ci
+        L.matmul_forward_splitk_forced_status.argtypes = [vp] * 4 + [ci] * 5 + [vp, cz] + [ci] * 3
+        L.matmul_forward_splitk_forced_status.restype = ci
+        L.matmul_forward_splitk_plan.argtypes = [ci] * 4 + [cz] + [ctypes.POINTER(ci)] * 3
+        L.matmul_forward_splitk_plan.restype = ci
         L.gpt2_create.argtypes, L.gpt2_create.restype = [ctypes.POINTER(GPT2Config)], vp
         L.gpt2_destroy.argtypes, L.gpt2_destroy.restype = [vp], None
         L.gpt2_checkpoint_read_config.argtypes = [ctypes.c_char_p, ctypes.POINTER(GPT2Config)]
@@ -277,6 +287,40 @@ def matmul_forward_tile_shape(B, T, C, OC):
     _check(lib().matmul_forward_tile_shape(B, T, C, OC, ctypes.byref(bm), ctypes.byref(bn)),
            "matmul_forward_tile_shape")
     return bm.value, bn.value
+
+
+SPLITK_COUNTER_BYTES = 16384
+
+
+def matmul_forward_splitk_workspace():
+    """A zero-filled workspace (uint8 CUDA tensor) of the size the library recommends."""
+    import torch
+    return torch.zeros(lib().matmul_forward_splitk_workspace(), dtype=torch.uint8, device="cuda")
+
+
+def matmul_forward_splitk(out, inp, weight, bias, B, T, C, OC, workspace, is_gelu=False, plan=None):
+    """matmul_forward_gelu with a workspace that lets K be split between workgroups.
+    workspace: uint8 CUDA tensor whose first SPLITK_COUNTER_BYTES were zero before its first
+    use.  plan: optional (tile_rows, tile_cols, splits) to force instead of the cost model's."""
+    ws, nbytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel())
+    if plan is None:
+        _check(lib().matmul_forward_splitk_status(_f32(out), _f32(inp), _f32(weight), _f32(bias), B,
+                                                  T, C, OC, int(bool(is_gelu)), ws, nbytes),
+               "matmul_forward_splitk")
+    else:
+        _check(lib().matmul_forward_splitk_forced_status(_f32(out), _f32(inp), _f32(weight),
+                                                         _f32(bias), B, T, C, OC, int(bool(is_gelu)),
+                                                         ws, nbytes, *map(int, plan)),
+               "matmul_forward_splitk_forced")
+
+
+def matmul_forward_splitk_plan(B, T, C, OC, workspace_bytes):
+    """(tile_rows, tile_cols, splits) that matmul_forward_splitk would use.  No GPU needed."""
+    bm, bn, sp = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    _check(lib().matmul_forward_splitk_plan(B, T, C, OC, workspace_bytes, ctypes.byref(bm),
+                                            ctypes.byref(bn), ctypes.byref(sp)),
+           "matmul_forward_splitk_plan")
+    return bm.value, bn.value, sp.value
 
 
 def attention_forward(out, qkvr, att, inp, B, T, C, NH):

@@ -55,31 +55,6 @@ constexpr int LDS_BAD = LDS_SMALL + 32;                   // one int: a wait tim
 constexpr int LDS_FREE = LDS_BAD + 32;
 
 
-// ---- cache-bypassing accesses for data that other workgroups wrote in this launch ---------
-// 128-bit ones go through buffer instructions, whose builtins take the cache policy (sc0 sc1)
-// and leave the bookkeeping of loads in flight to the compiler.
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-constexpr int kBypass = 0x11;  // sc0 | sc1
-struct Bypass {
-  __amdgpu_buffer_rsrc_t rsrc;
-  __device__ __forceinline__ Bypass(const float* base, size_t floats)
-      : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)(floats * sizeof(float)),
-                                               0x00020000)) {}
-  // float_index: this lane's first float (reads past `floats` return zero)
-  __device__ __forceinline__ f32x4 load4(int float_index) const {
-    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, float_index * 4, 0, kBypass));
-  }
-  __device__ __forceinline__ void store4(int float_index, f32x4 v) const {
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, float_index * 4, 0, kBypass);
-  }
-};
-__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
-__device__ __forceinline__ float load_bypass(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void store_bypass(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 // Layout of the activations that one phase writes and every workgroup reads in the next (the
 // residual stream x, the attention output, the MLP's hidden row): granules of 4 sequences x 4
 // channels, [sequence / 4][channel / 4][sequence % 4][channel % 4], always 4 * JG sequences

@@ -53,6 +53,8 @@ struct GPT2 {
   float* logits;   // (M,V)
   void* pairs;     // workspace of matmul_forward_argmax for (M,V)
   size_t pairs_bytes;
+  void* splitk;    // workspace of matmul_forward_splitk: counters (zero between calls) + partial tiles
+  size_t splitk_bytes;
   int last_B, last_T;
   bool last_has_logits;
 
@@ -99,13 +101,13 @@ static void drop_graphs(GPT2* m) {
 static void free_activations(GPT2* m) {
   drop_graphs(m);
   void* ptrs[] = {m->ids,  m->res_a, m->res_b, m->ln,     m->qkv,
-                  m->atty, m->proj,  m->fch,   m->logits, m->pairs};
+                  m->atty, m->proj,  m->fch,   m->logits, m->pairs, m->splitk};
   for (void* p : ptrs)
     if (p) (void)hipFree(p);
   m->ids = nullptr;
   m->res_a = m->res_b = m->ln = m->qkv = m->atty = m->proj = m->fch = m->logits = nullptr;
-  m->pairs = nullptr;
-  m->pairs_bytes = 0;
+  m->pairs = m->splitk = nullptr;
+  m->pairs_bytes = m->splitk_bytes = 0;
   m->cap_tokens = 0;
 }
 
@@ -172,7 +174,8 @@ static int reserve(GPT2* m, int B, int T) {
       {(void**)&m->qkv, n * 3 * C * 4},            {(void**)&m->atty, n * C * 4},
       {(void**)&m->proj, n * C * 4},               {(void**)&m->fch, n * 4 * C * 4},
       {(void**)&m->logits, n * V * 4},
-      {&m->pairs, matmul_forward_argmax_workspace(1, (int)M, (int)V)}};
+      {&m->pairs, matmul_forward_argmax_workspace(1, (int)M, (int)V)},
+      {&m->splitk, matmul_forward_splitk_workspace()}};
   for (auto& w : want) {
     hipError_t e = hipMalloc(w.p, w.bytes);
     if (e != hipSuccess) {
@@ -183,6 +186,12 @@ static int reserve(GPT2* m, int B, int T) {
     }
   }
   m->pairs_bytes = matmul_forward_argmax_workspace(1, (int)M, (int)V);
+  // the counters start at zero; every GEMM that uses them leaves them at zero
+  if (hipMemset(m->splitk, 0, GPT2HIP_SPLITK_COUNTER_BYTES) != hipSuccess) {
+    free_activations(m);
+    return fail(GPT2HIP_EHIP, "gpt2: clearing the K-split counters failed");
+  }
+  m->splitk_bytes = matmul_forward_splitk_workspace();
   m->cap_tokens = M;
   return GPT2HIP_OK;
 }
@@ -263,25 +272,27 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
   G2_STEP(GPT2_PROF_ENCODER, encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE), B, T, C, V));
   // the one stand-alone layernorm: ln1 of layer 0
   G2_STEP(GPT2_PROF_LAYERNORM, layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, T, C));
+  // The four GEMMs of a block may split K between workgroups through the model's workspace
+  // (short prompts, where a layer has fewer tiles than the device has compute units).
   for (int l = 0; l < L; l++) {
-    G2_STEP(GPT2_PROF_MATMUL_QKV, matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
-                                 B, T, C, 3 * C));
+    G2_STEP(GPT2_PROF_MATMUL_QKV, matmul_forward_splitk_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
+                                 B, T, C, 3 * C, 0, m->splitk, m->splitk_bytes));
     if (fill_cache) {
       const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
       G2_TRY(kv_store_launch(m->kv + (2 * (size_t)l) * plane, m->kv + (2 * (size_t)l + 1) * plane, m->qkv,
                              B, T, c.max_seq_len, C, NH));
     }
     G2_STEP(GPT2_PROF_ATTENTION, attention_forward_status(m->atty, nullptr, nullptr, m->qkv, B, T, C, NH));
-    G2_STEP(GPT2_PROF_MATMUL_ATTPROJ, matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs,
-                                 P(P_ATTPROJB) + l * cs, B, T, C, C));
+    G2_STEP(GPT2_PROF_MATMUL_ATTPROJ, matmul_forward_splitk_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs,
+                                 P(P_ATTPROJB) + l * cs, B, T, C, C, 0, m->splitk, m->splitk_bytes));
     // residual2 = residual + attproj ; ln = ln2(residual2)
     G2_STEP(GPT2_PROF_FUSED_RESIDUAL_LAYERNORM, fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual,
                                                    m->proj, P(P_LN2W) + l * cs, P(P_LN2B) + l * cs,
                                                    B, T, C));
-    G2_STEP(GPT2_PROF_MATMUL_FC_GELU, matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs,
-                                      P(P_FCB) + l * 4 * cs, B, T, C, 4 * C, 1));
-    G2_STEP(GPT2_PROF_MATMUL_FCPROJ, matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
-                                 P(P_FCPROJB) + l * cs, B, T, 4 * C, C));
+    G2_STEP(GPT2_PROF_MATMUL_FC_GELU, matmul_forward_splitk_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs,
+                                      P(P_FCB) + l * 4 * cs, B, T, C, 4 * C, 1, m->splitk, m->splitk_bytes));
+    G2_STEP(GPT2_PROF_MATMUL_FCPROJ, matmul_forward_splitk_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
+                                 P(P_FCPROJB) + l * cs, B, T, 4 * C, C, 0, m->splitk, m->splitk_bytes));
     // residual3 = residual2 + fcproj ; ln = ln1 of the next layer, or the final layernorm
     const float* nw = (l + 1 < L) ? P(P_LN1W) + (l + 1) * cs : P(P_LNFW);
     const float* nb = (l + 1 < L) ? P(P_LN1B) + (l + 1) * cs : P(P_LNFB);

@@ -105,6 +105,75 @@ __device__ __forceinline__ void argmax_fold(float* bv, int* bx, int lane, int& f
   }
 }
 
+// K split between workgroups.  The `splits` workgroups of a tile each multiply one
+// contiguous range of the K slabs and leave their partial tile (the raw accumulators, lane
+// by lane: [tile][part][wave][register quad][lane], 1 KB per store instruction) in a
+// workspace; whichever of them finishes last -- a per-tile counter tells it, nobody ever
+// waits -- reads all the parts back IN PART ORDER into its accumulators and runs the
+// ordinary epilogue, so the result does not depend on which workgroup that was.  The
+// partial tiles cross XCDs: they are stored and loaded with the cache-bypassing policy,
+// each wave waits for its stores to be acknowledged before the workgroup counts itself
+// in, and the last one resets the counter for the next launch.
+// Returns false in the workgroups that are done (everyone but the tile's last one).
+template <int NW, int TM, int TN>
+__device__ __forceinline__ bool splitk_combine(f32x16 (&acc)[TM][TN], float* __restrict__ part_ws,
+                                               unsigned* __restrict__ part_cnt, int tile_id, int part,
+                                               int splits, int slot, bool holds, int lane, int tid,
+                                               int* lds_flag) {
+  constexpr int ACC4 = TM * TN * 4;             // register quads per lane
+  constexpr int PART_FLOATS = NW * ACC4 * 256;  // one partial tile
+  const Bypass ws(part_ws + (size_t)tile_id * splits * PART_FLOATS, (size_t)splits * PART_FLOATS);
+  if (holds) {
+    const int mine = (part * NW + slot) * (ACC4 * 256) + lane * 4;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const f32x4 q = {acc[i][j][4 * u], acc[i][j][4 * u + 1], acc[i][j][4 * u + 2],
+                           acc[i][j][4 * u + 3]};
+          ws.store4(mine + ((i * TN + j) * 4 + u) * 256, q);
+        }
+  }
+  wait_vm();
+  __syncthreads();
+  if (tid == 0) {
+    const unsigned old =
+        __hip_atomic_fetch_add(part_cnt + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = old + 1u == (unsigned)splits;
+    if (last) __hip_atomic_store(part_cnt + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *lds_flag = last ? 1 : 0;
+  }
+  __syncthreads();
+  if (*lds_flag == 0 || !holds) return false;
+  // Four parts at a time, all their loads independent of each other so that as many are in
+  // flight as the registers allow; a part past the last one lies beyond the end of the
+  // buffer descriptor and reads as zeros without touching memory.
+  for (int p0 = 0; p0 < splits; p0 += 4) {
+    f32x4 t[4][ACC4];
+#pragma unroll
+    for (int pp = 0; pp < 4; pp++) {
+      const int theirs = ((p0 + pp) * NW + slot) * (ACC4 * 256) + lane * 4;
+#pragma unroll
+      for (int q = 0; q < ACC4; q++) t[pp][q] = ws.load4(theirs + q * 256);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int q = (i * TN + j) * 4 + (v >> 2);
+          float x = p0 == 0 ? t[0][q][v & 3] : acc[i][j][v] + t[0][q][v & 3];
+#pragma unroll
+          for (int pp = 1; pp < 4; pp++) x += t[pp][q][v & 3];
+          acc[i][j][v] = x;
+        }
+  }
+  return true;
+}
+
 template <int BM, int BN, int WGM, int WGN, bool GELU, bool KTAIL>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
@@ -349,11 +418,16 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 // one (largest value, its column) pair and stores that in out[row][tn * WGN + wn] (the
 // value) and arg_idx[row][tn * WGN + wn] (the column): ntn * WGN pairs per row, which
 // argmax_pairs_kernel reduces.  The (M, N) product itself never reaches memory.
-template <int BM, int BN, int WGM, int WGN, bool GELU, bool PROBE = false, bool ARGMAX = false>
+//
+// SPLIT: the grid is `splits` workgroups per tile (workgroup id = part * tiles + tile), each
+// taking slabs [part * nslab / splits, (part + 1) * nslab / splits); see splitk_combine.
+template <int BM, int BN, int WGM, int WGN, bool GELU, bool PROBE = false, bool ARGMAX = false,
+          bool SPLIT = false>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
     const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn,
-    unsigned long long* __restrict__ probe, int* __restrict__ arg_idx) {
+    unsigned long long* __restrict__ probe, int* __restrict__ arg_idx, float* __restrict__ part_ws,
+    unsigned* __restrict__ part_cnt, int splits) {
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -373,9 +447,17 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
 
+  int pid = blockIdx.x, part = 0;
+  if (SPLIT) {
+    part = pid / (ntm * ntn);
+    pid -= part * (ntm * ntn);
+  }
   int tm, tn;
-  tile_of_block(blockIdx.x, ntm, ntn, tm, tn);
+  tile_of_block(pid, ntm, ntn, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
+  // this workgroup's slabs: all of K, or its part of it
+  const int slab_lo = SPLIT ? (int)((long long)part * (K / BK) / splits) : 0;
+  const int nslab = SPLIT ? (int)((long long)(part + 1) * (K / BK) / splits) - slab_lo : K / BK;
 
   // ---- LDS-DMA descriptors -------------------------------------------------
   // One DMA fills a group of 8 rows of a buffer.  Each wave owns A_PER groups of the A
@@ -386,8 +468,8 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   // per-lane byte offset, so the loop spends no vector instructions on addressing.
   constexpr int A_PER = BM / 8 / NW, B_PER = BN / 8 / NW;
   static_assert(BM / 8 % NW == 0 && BN / 8 % NW == 0, "tile/waves mismatch");
-  const char* const a_tile = reinterpret_cast<const char*>(inp + (size_t)m0 * K);
-  const char* const b_tile = reinterpret_cast<const char*>(weight + (size_t)n0 * K);
+  const char* const a_tile = reinterpret_cast<const char*>(inp + (size_t)m0 * K + (size_t)slab_lo * BK);
+  const char* const b_tile = reinterpret_cast<const char*>(weight + (size_t)n0 * K + (size_t)slab_lo * BK);
   unsigned dma_off[DMA_PER];
   int dma_group[DMA_PER];  // wave-uniform: which 8-row group of the buffer
   {
@@ -405,7 +487,6 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
       }
     }
   }
-  const int nslab = K / BK;
   auto dma_slab = [&](int slab, int buf) {
     const size_t kbytes = (size_t)min(slab, nslab - 1) * (BK * 4);  // past the end: reload
     const char* a_k = a_tile + kbytes;
@@ -424,12 +505,13 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   dma_slab(0, 0);
   dma_slab(1, 1);
 
-  // ---- accumulators, initialised with the bias of the lane's column ----
+  // ---- accumulators, initialised with the bias of the lane's column (in the part that
+  // takes the first slabs, when K is split) ----
   f32x16 acc[TM][TN];
 #pragma unroll
   for (int j = 0; j < TN; j++) {
     const int col = n0 + wn * WN + j * 32 + (lane & 31);
-    const float bv = (bias != nullptr && col < N) ? bias[col] : 0.f;
+    const float bv = (bias != nullptr && col < N && part == 0) ? bias[col] : 0.f;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -534,6 +616,13 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
 #undef G2_SGB
 #undef G2_READS_IN_SHADOW
 
+  if constexpr (SPLIT) {
+    __syncthreads();  // every wave has finished with the LDS buffers: word 0 becomes the flag
+    if (!splitk_combine<NW, TM, TN>(acc, part_ws, part_cnt, pid, part, splits, wave, true, lane, tid,
+                                    reinterpret_cast<int*>(lds_bytes)))
+      return;
+  }
+
   // ---- epilogue -----------------------------------------------------------
   if (ARGMAX) {
     const size_t pairs = (size_t)ntn * WGN;
@@ -618,10 +707,12 @@ constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 // slab, so a 32x32 tile still keeps all four SIMDs of its CU busy.  The partial
 // accumulators are summed through LDS in a fixed order (ks = 0, 1, ...), so results do
 // not depend on timing.
-template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool GELU>
+// SPLIT: K is also split between `splits` workgroups per tile, as in matmul_dma_kernel.
+template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool GELU, bool SPLIT = false>
 __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn) {
+    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn,
+    float* __restrict__ part_ws, unsigned* __restrict__ part_cnt, int splits) {
   constexpr int NMN = WGM * WGN;
   constexpr int NW = NMN * KS;
   constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -646,13 +737,20 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
   const int ks = wave / NMN, wmn = wave % NMN;
   const int wm = wmn / WGN, wn = wmn % WGN;
 
+  int pid = blockIdx.x, part = 0;
+  if (SPLIT) {
+    part = pid / (ntm * ntn);
+    pid -= part * (ntm * ntn);
+  }
   int tm, tn;
-  tile_of_block(blockIdx.x, ntm, ntn, tm, tn);
+  tile_of_block(pid, ntm, ntn, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
+  const int slab_lo = SPLIT ? (int)((long long)part * (K / BK) / splits) : 0;
+  const int nslab = SPLIT ? (int)((long long)(part + 1) * (K / BK) / splits) - slab_lo : K / BK;
 
   // LDS-DMA descriptors, as in matmul_dma_kernel
-  const char* const a_tile = reinterpret_cast<const char*>(inp + (size_t)m0 * K);
-  const char* const b_tile = reinterpret_cast<const char*>(weight + (size_t)n0 * K);
+  const char* const a_tile = reinterpret_cast<const char*>(inp + (size_t)m0 * K + (size_t)slab_lo * BK);
+  const char* const b_tile = reinterpret_cast<const char*>(weight + (size_t)n0 * K + (size_t)slab_lo * BK);
   unsigned dma_off[DMA_PER];
   int dma_group[DMA_PER];
   {
@@ -670,7 +768,6 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
       }
     }
   }
-  const int nslab = K / BK;
   auto dma_slab = [&](int slab, int buf) {
     const size_t kbytes = (size_t)min(slab, nslab - 1) * (BK * 4);  // past the end: reload
     const char* a_k = a_tile + kbytes;
@@ -690,7 +787,7 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
 #pragma unroll
   for (int j = 0; j < TN; j++) {
     const int col = n0 + wn * WN + j * 32 + (lane & 31);
-    const float bv = (bias != nullptr && ks == 0 && col < N) ? bias[col] : 0.f;
+    const float bv = (bias != nullptr && ks == 0 && part == 0 && col < N) ? bias[col] : 0.f;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -752,17 +849,25 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
                 acc[i][j][v];
     }
     __syncthreads();
-    if (ks > 0) return;
+    if (!SPLIT && ks > 0) return;
+    if (ks == 0) {
 #pragma unroll
-    for (int k2 = 1; k2 < KS; k2++)
+      for (int k2 = 1; k2 < KS; k2++)
 #pragma unroll
-      for (int i = 0; i < TM; i++)
+        for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
+          for (int j = 0; j < TN; j++)
 #pragma unroll
-          for (int v = 0; v < 16; v++)
-            acc[i][j][v] +=
-                red[((((k2 - 1) * NMN + wmn) * (TM * TN) + i * TN + j) * 16 + v) * 64 + lane];
+            for (int v = 0; v < 16; v++)
+              acc[i][j][v] +=
+                  red[((((k2 - 1) * NMN + wmn) * (TM * TN) + i * TN + j) * 16 + v) * 64 + lane];
+    }
+  }
+  if constexpr (SPLIT) {
+    __syncthreads();  // the LDS is free: word 0 becomes the flag
+    if (!splitk_combine<NMN, TM, TN>(acc, part_ws, part_cnt, pid, part, splits, wmn, ks == 0, lane, tid,
+                                     reinterpret_cast<int*>(lds_bytes)))
+      return;
   }
 
   const bool full = (m0 + BM <= M) && (n0 + BN <= N);
@@ -1013,7 +1118,7 @@ __global__ __launch_bounds__(256) void matmul_argmax_generic_kernel(int* __restr
 // Raises the dynamic-LDS limit of a kernel, once per (thread, device, kernel).
 static int allow_lds(const void* kfn, size_t lds_bytes) {
   static thread_local int configured_for = -1;
-  static thread_local const void* configured[32];
+  static thread_local const void* configured[64];
   static thread_local int nconfigured = 0;
   int dev = 0;
   G2_HIP(hipGetDevice(&dev));
@@ -1024,7 +1129,7 @@ static int allow_lds(const void* kfn, size_t lds_bytes) {
   for (int i = 0; i < nconfigured; i++)
     if (configured[i] == kfn) return GPT2HIP_OK;
   G2_HIP(hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  if (nconfigured < 32) configured[nconfigured++] = kfn;
+  if (nconfigured < 64) configured[nconfigured++] = kfn;
   return GPT2HIP_OK;
 }
 
@@ -1049,24 +1154,36 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
   return GPT2HIP_OK;
 }
 
+// K split between the workgroups of a tile (splitk_combine): where the partial tiles and the
+// per-tile counters live, and how many parts.  splits == 1: no split.
+struct SplitK {
+  float* ws = nullptr;
+  unsigned* cnt = nullptr;
+  int splits = 1;
+};
+
 // LDS-DMA kernel: K % 32 == 0.  The clock-probe form exists for PROBED tile shapes only.
 template <int BM, int BN, int WGM, int WGN, bool PROBED = false>
 static int launch_dma(float* out, const float* inp, const float* weight, const float* bias, int M,
-                      int K, int N, bool gelu, unsigned long long* probe = nullptr) {
+                      int K, int N, bool gelu, unsigned long long* probe = nullptr, SplitK sk = {}) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
-  const long long tiles = (long long)ntm * ntn;
+  const long long tiles = (long long)ntm * ntn * sk.splits;
   if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
   auto kfn = gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true> : matmul_dma_kernel<BM, BN, WGM, WGN, false>;
-  if constexpr (PROBED) {
+  if (sk.splits > 1) {
+    if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: no probe form with K split");
+    kfn = gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true, false, false, true>
+               : matmul_dma_kernel<BM, BN, WGM, WGN, false, false, false, true>;
+  } else if constexpr (PROBED) {
     if (probe) kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, true>;
   } else if (probe) {
     return fail(GPT2HIP_EINVAL, "matmul_forward_probe: no probe form of the %dx%d tile", BM, BN);
   }
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
-                     K, N, ntm, ntn, probe, (int*)nullptr);
+                     K, N, ntm, ntn, probe, (int*)nullptr, sk.ws, sk.cnt, sk.splits);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1083,7 +1200,8 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
   auto kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, false, true>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)(ntm * ntn)), dim3(NT), lds_bytes, stream(), pair_val, inp, weight,
-                     bias, M, K, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx);
+                     bias, M, K, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx, (float*)nullptr,
+                     (unsigned*)nullptr, 1);
   G2_LAUNCH_CHECK("matmul_forward_argmax");
   hipLaunchKernelGGL(argmax_pairs_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, stream(), ids,
                      pair_val, pair_idx, M, ntn * WGN);
@@ -1094,17 +1212,20 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
 // Ring kernel for small problems: K % 32 == 0.
 template <int BM, int BN, int WGM, int WGN, int KS, int NBUF>
 static int launch_ring(float* out, const float* inp, const float* weight, const float* bias, int M,
-                       int K, int N, bool gelu) {
+                       int K, int N, bool gelu, SplitK sk = {}) {
   constexpr int NT = WGM * WGN * KS * kWave;
   constexpr size_t lds_bytes = (size_t)NBUF * (BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
-  const long long tiles = (long long)ntm * ntn;
+  const long long tiles = (long long)ntm * ntn * sk.splits;
   if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
   auto kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true>
                   : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false>;
+  if (sk.splits > 1)
+    kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true, true>
+               : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false, true>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
-                     K, N, ntm, ntn);
+                     K, N, ntm, ntn, sk.ws, sk.cnt, sk.splits);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1125,41 +1246,129 @@ struct TileChoice {
   int index;        // into the candidate list below
   int bm, bn;
   long long tiles;
+  int splits;       // workgroups per tile (K split between them), 1 = none
 };
-static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only) {
-  struct Cand { int bm, bn; double a, round_us, launch_us; };
-  // (64x192 and 128x64 were fitted too -- a = 1.033 and 1.042 -- and never won by more than
-  // 0.4 % anywhere in the sweep: not built)
-  const Cand cands[] = {{128, 192, 0.988, 6.42, -2.15}, {128, 128, 1.006, 3.59, -0.11},
-                        {128, 96, 1.017, 1.84, 1.93},   {64, 128, 1.042, 2.08, 1.01},
-                        {64, 64, 1.159, 0.40, 1.88},    {32, 32, 1.398, 0.0, 3.54}};
-  constexpr int kCands = (int)(sizeof(cands) / sizeof(cands[0]));
-  constexpr double kCuFlopsPerUs = 579e3;  // what one compute unit sustains in the 128x192 loop
-  int best = 0;
-  double best_cost = 0;
-  long long best_tiles = 0;
-  for (int i = 0; i < (two_largest_only ? 2 : kCands); i++) {
-    const long long t = (long long)((M + cands[i].bm - 1) / cands[i].bm) *
-                        ((OC + cands[i].bn - 1) / cands[i].bn);
-    Cand c = cands[i];
-    if (i == 4 && t <= 2 * 256) c = Cand{64, 64, 1.190, 0.35, 2.98};  // the ring form of 64x64
+// fix_*: what a K split between workgroups adds (fitted per shape to a second forced sweep, over
+// 2..8 parts): fix_us + fix_part_us x parts + fix_mb_us x MB of partial tiles.  The partial
+// tiles cross memory twice (parts x the size of the product each way), which is what makes a
+// split pay at K = 3072 or 4096 (up to 20 %, twice as fast at B*T <= 128) and hardly ever at
+// K = 768, where that traffic costs as much as the rounds it fills.
+struct TileCand { int bm, bn; double a, round_us, launch_us, fix_us, fix_part_us, fix_mb_us; };
+// (64x192 and 128x64 were fitted too -- a = 1.033 and 1.042 -- and never won by more than
+// 0.4 % anywhere in the sweep: not built)
+static const TileCand kTileCands[] = {
+    {128, 192, 0.988, 6.42, -2.15, 4.21, 0.90, 0.069}, {128, 128, 1.006, 3.59, -0.11, 3.81, 0.64, 0.022},
+    {128, 96, 1.017, 1.84, 1.93, 2.73, 0.54, 0.067},   {64, 128, 1.042, 2.08, 1.01, 2.48, 0.43, 0.0},
+    {64, 64, 1.159, 0.40, 1.88, 1.68, 0.21, 0.116},    {32, 32, 1.398, 0.0, 3.54, 0.90, 0.19, 0.468}};
+// a split is taken when the model puts it this far ahead of the best plan without one (over
+// the sweep no chosen split is then slower than that plan; 0.9 % behind the best forced plan
+// on average, 5.8 % ahead of the choice without splits)
+constexpr double kSplitMargin = 1.08;
+constexpr int kTileCandCount = (int)(sizeof(kTileCands) / sizeof(kTileCands[0]));
+constexpr double kCuFlopsPerUs = 579e3;  // what one compute unit sustains in the 128x192 loop
+constexpr size_t kSplitCounters = GPT2HIP_SPLITK_COUNTER_BYTES / sizeof(unsigned);
+
+static long long tiles_of(int i, int M, int OC) {
+  return (long long)((M + kTileCands[i].bm - 1) / kTileCands[i].bm) *
+         ((OC + kTileCands[i].bn - 1) / kTileCands[i].bn);
+}
+
+// Whether `splits` workgroups per tile of candidate i fit the workspace (counters first, then
+// tiles x splits partial tiles) and the kernel (every part needs a slab).
+static bool split_fits(int i, int M, int C, int OC, int splits, size_t workspace_bytes) {
+  if (splits == 1) return true;
+  const long long t = tiles_of(i, M, OC);
+  if (splits < 1 || splits > C / BK || t > (long long)kSplitCounters) return false;
+  if (workspace_bytes < GPT2HIP_SPLITK_COUNTER_BYTES) return false;
+  const unsigned long long need =
+      (unsigned long long)t * splits * kTileCands[i].bm * kTileCands[i].bn * sizeof(float);
+  return need <= workspace_bytes - GPT2HIP_SPLITK_COUNTER_BYTES;
+}
+
+// workspace_bytes == 0: no K split between workgroups.
+static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only, size_t workspace_bytes = 0) {
+  int best = 0, split_best = -1, split_parts = 1;
+  double best_cost = 0, split_cost = 0;
+  for (int i = 0; i < (two_largest_only ? 2 : kTileCandCount); i++) {
+    const long long t = tiles_of(i, M, OC);
+    TileCand c = kTileCands[i];
     const double work_us = 2.0 * c.bm * c.bn * (double)C / kCuFlopsPerUs;
-    const double cost = c.launch_us + (double)((t + 255) / 256) * (c.a * work_us + c.round_us);
-    if (i == 0 || cost < best_cost) {
-      best = i;
-      best_cost = cost;
-      best_tiles = t;
+    // K split S ways: S times the workgroups, each with 1/S of the matrix work, plus the
+    // partial tiles' trip through memory (written once, read once by the last arrival)
+    for (int S = 1; S <= 8; S++) {
+      if (S > 1 && (workspace_bytes == 0 || two_largest_only || t * S > 6 * 256 ||
+                    !split_fits(i, M, C, OC, S, workspace_bytes)))
+        continue;
+      TileCand k = c;
+      if (i == 4 && t * S <= 2 * 256) {  // the ring form of 64x64
+        k.a = 1.190;
+        k.round_us = 0.35;
+        k.launch_us = 2.98;
+      }
+      double cost = k.launch_us + (double)((t * S + 255) / 256) * (k.a * work_us / S + k.round_us);
+      if (S == 1) {
+        if (i == 0 || cost < best_cost) {
+          best = i;
+          best_cost = cost;
+        }
+      } else {
+        cost += k.fix_us + k.fix_part_us * S + k.fix_mb_us * ((double)t * S * k.bm * k.bn * 4e-6);
+        if (split_best < 0 || cost < split_cost) {
+          split_best = i;
+          split_cost = cost;
+          split_parts = S;
+        }
+      }
     }
     // sixteen or more rounds of the largest tile (the lm-head): rounding up to whole
     // rounds costs at most 3 %, less than any smaller tile loses
     if (i == 0 && t >= 16 * 256) break;
   }
-  return TileChoice{best, cands[best].bm, cands[best].bn, best_tiles};
+  if (split_best >= 0 && split_cost * kSplitMargin < best_cost)
+    return TileChoice{split_best, kTileCands[split_best].bm, kTileCands[split_best].bn,
+                      tiles_of(split_best, M, OC), split_parts};
+  return TileChoice{best, kTileCands[best].bm, kTileCands[best].bn, tiles_of(best, M, OC), 1};
 }
 
+// Launches candidate `best` with the K split of `sk`.
+static int launch_choice(int best, long long best_tiles, float* out, const float* inp, const float* weight,
+                         const float* bias, int M, int C, int OC, bool gelu, unsigned long long* probe,
+                         SplitK sk) {
+  switch (best) {
+    case 5:
+      // one 32x32 tile per workgroup, its four waves splitting K
+      return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu, sk);
+    case 4:
+      // up to two workgroups per CU: latency-bound, ring of four slabs and a 2-way K split
+      if (best_tiles * sk.splits <= 2 * 256)
+        return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu, sk);
+      return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+    case 3:
+      return launch_dma<64, 128, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+    case 2:
+      // four waves of 32x96: two workgroups per compute unit
+      return launch_dma<128, 96, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+    case 1:
+      return launch_dma<128, 128, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk);
+    default:
+      // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
+      // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
+      // gives every SIMD two waves to alternate between.
+      if (best_tiles >= 16 * 256 && sk.splits == 1)
+        return launch_dma<128, 192, 2, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
+      return launch_dma<128, 192, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk);
+  }
+}
+
+// workspace (optional): GPT2HIP_SPLITK_COUNTER_BYTES of counters that are zero between calls,
+// then room for partial tiles; allows K to be split between workgroups.  forced (optional):
+// a tile shape and split count to use instead of the cost model's.
+struct ForcedPlan { int bm, bn, splits; };
 static int matmul_dispatch(float* out, const float* inp, const float* weight, const float* bias,
                            int B, int T, int C, int OC, bool gelu,
-                           unsigned long long* probe = nullptr, int* probe_groups = nullptr) {
+                           unsigned long long* probe = nullptr, int* probe_groups = nullptr,
+                           void* workspace = nullptr, size_t workspace_bytes = 0,
+                           const ForcedPlan* forced = nullptr) {
   if (B < 0 || T < 0 || C < 1 || OC < 1)
     return fail(GPT2HIP_EINVAL, "matmul_forward: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
   const long long M64 = (long long)B * T;
@@ -1167,6 +1376,12 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
   const int M = (int)M64;
   if (M == 0) return GPT2HIP_OK;
   if (!out || !inp || !weight) return fail(GPT2HIP_EINVAL, "matmul_forward: null pointer");
+  if (workspace && ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0))
+    return fail(GPT2HIP_EINVAL, "matmul_forward: workspace must be 256-byte aligned");
+  if (!workspace) workspace_bytes = 0;
+  const bool tiled = C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31) && C % 4 == 0 &&
+                     aligned16(inp) && aligned16(weight);
+  if (forced && !tiled) return fail(GPT2HIP_EINVAL, "matmul_forward: a forced plan needs C %% 32 == 0 and aligned operands");
   if (C % 4 != 0 || !aligned16(inp) || !aligned16(weight)) {
     if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs the MFMA path");
     const size_t total = (size_t)M * OC;
@@ -1175,39 +1390,32 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
     G2_LAUNCH_CHECK("matmul_forward");
     return GPT2HIP_OK;
   }
-  if (M <= 16 && C % 16 == 0 && !probe)
+  if (M <= 16 && C % 16 == 0 && !probe && !forced)
     return skinny_launch(out, inp, weight, bias, nullptr, nullptr, nullptr, M, C, OC, gelu);
   // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
-  if (C % BK == 0 && (long long)C * 192 * 4 < (1LL << 31)) {
-    const TileChoice choice = choose_tile(M, C, OC, probe != nullptr);
-    const int best = choice.index;
-    const long long best_tiles = choice.tiles;
-    if (best_tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
-    if (probe_groups) *probe_groups = (int)best_tiles;
-    switch (best) {
-      case 5:
-        // one 32x32 tile per workgroup, its four waves splitting K
-        return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu);
-      case 4:
-        // up to two tiles per CU: latency-bound, ring of four slabs and a 2-way K split
-        if (best_tiles <= 2 * 256)
-          return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu);
-        return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu);
-      case 3:
-        return launch_dma<64, 128, 2, 2>(out, inp, weight, bias, M, C, OC, gelu);
-      case 2:
-        // four waves of 32x96: two workgroups per compute unit
-        return launch_dma<128, 96, 4, 1>(out, inp, weight, bias, M, C, OC, gelu);
-      case 1:
-        return launch_dma<128, 128, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
-      default:
-        // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
-        // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
-        // gives every SIMD two waves to alternate between.
-        if (best_tiles >= 16 * 256)
-          return launch_dma<128, 192, 2, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
-        return launch_dma<128, 192, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
+  if (tiled) {
+    TileChoice choice;
+    if (forced) {
+      int idx = -1;
+      for (int i = 0; i < kTileCandCount; i++)
+        if (kTileCands[i].bm == forced->bm && kTileCands[i].bn == forced->bn) idx = i;
+      if (idx < 0) return fail(GPT2HIP_EINVAL, "matmul_forward: no %dx%d tile", forced->bm, forced->bn);
+      if (!split_fits(idx, M, C, OC, forced->splits, workspace_bytes))
+        return fail(GPT2HIP_EINVAL, "matmul_forward: %d-way K split of %dx%d tiles does not fit (K slabs %d, workspace %zu bytes)",
+                    forced->splits, forced->bm, forced->bn, C / BK, workspace_bytes);
+      choice = TileChoice{idx, forced->bm, forced->bn, tiles_of(idx, M, OC), forced->splits};
+    } else {
+      choice = choose_tile(M, C, OC, probe != nullptr, workspace_bytes);
     }
+    if (choice.tiles * choice.splits > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
+    if (probe_groups) *probe_groups = (int)choice.tiles;
+    SplitK sk;
+    if (choice.splits > 1) {
+      sk.cnt = static_cast<unsigned*>(workspace);
+      sk.ws = reinterpret_cast<float*>(static_cast<char*>(workspace) + GPT2HIP_SPLITK_COUNTER_BYTES);
+      sk.splits = choice.splits;
+    }
+    return launch_choice(choice.index, choice.tiles, out, inp, weight, bias, M, C, OC, gelu, probe, sk);
   }
   if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs C %% 32 == 0");
   return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu);
@@ -1337,6 +1545,45 @@ int matmul_forward_argmax_noalloc_status(int* ids, const float* inp, const float
   void* ptr = nullptr;
   if (int rc = scratch_address(&ptr)) return rc;
   return argmax_dispatch(ids, ptr, sizeof(scratch), inp, weight, bias, B, T, C, OC);
+}
+
+size_t matmul_forward_splitk_workspace(void) {
+  // counters + 512 partial tiles of the largest shape (two per compute unit)
+  return GPT2HIP_SPLITK_COUNTER_BYTES + (size_t)512 * 128 * 192 * sizeof(float);
+}
+
+int matmul_forward_splitk_status(float* out, const float* inp, const float* weight, const float* bias,
+                                 int B, int T, int C, int OC, int is_gelu, void* workspace,
+                                 size_t workspace_bytes) {
+  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, is_gelu != 0, nullptr, nullptr,
+                             workspace, workspace_bytes);
+}
+
+int matmul_forward_splitk_forced_status(float* out, const float* inp, const float* weight,
+                                        const float* bias, int B, int T, int C, int OC, int is_gelu,
+                                        void* workspace, size_t workspace_bytes, int tile_rows,
+                                        int tile_cols, int splits) {
+  const g2::ForcedPlan plan{tile_rows, tile_cols, splits};
+  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, is_gelu != 0, nullptr, nullptr,
+                             workspace, workspace_bytes, &plan);
+}
+
+int matmul_forward_splitk_plan(int B, int T, int C, int OC, size_t workspace_bytes, int* tile_rows,
+                               int* tile_cols, int* splits) {
+  using namespace g2;
+  const long long M64 = (long long)B * T;
+  if (B < 1 || T < 1 || C < 1 || OC < 1 || M64 > 0x7fffffffLL || !tile_rows || !tile_cols || !splits)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_splitk_plan: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
+  if (C % BK != 0 || M64 <= 16 || (long long)C * 192 * 4 >= (1LL << 31)) {
+    *tile_rows = *tile_cols = 0;  // not one of the tiled LDS-DMA kernels
+    *splits = 1;
+    return GPT2HIP_OK;
+  }
+  const TileChoice c = choose_tile((int)M64, C, OC, false, workspace_bytes);
+  *tile_rows = c.bm;
+  *tile_cols = c.bn;
+  *splits = c.splits;
+  return GPT2HIP_OK;
 }
 
 int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,

@@ -97,6 +97,38 @@ int matmul_forward_gelu_status(float* out, const float* inp, const float* weight
 void matmul_forward_gelu(float* out, const float* inp, const float* weight, const float* bias,
                          int B, int T, int C, int OC, int is_gelu);
 
+/* matmul_forward_gelu for a caller that can lend a workspace: with it the K dimension of a
+ * tile can be split between several workgroups, whose partial tiles meet in the workspace and
+ * are summed in a fixed order by whichever workgroup of the tile finishes last (results do not
+ * depend on timing; they differ from matmul_forward's by fp32 rounding of the summation
+ * order).  This is what fills the 256 compute units when a problem has too few tiles, or a
+ * tile count just above a multiple of 256 -- the "wave quantisation" that the reference's
+ * fixed grid of one 128x128 tile per block leaves in place
+ * (kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:266-274).  Whether and how K is split is
+ * chosen by the same fitted cost model as the tile shape; without a workspace (NULL / 0) the
+ * call is matmul_forward_gelu.
+ * workspace: device memory, 256-byte aligned.  Its first GPT2HIP_SPLITK_COUNTER_BYTES are
+ * per-tile counters: zero them once (hipMemset) before the first call; every call leaves them
+ * zero.  The rest holds partial tiles (tiles x splits x tile area x 4 bytes; a plan that does
+ * not fit is not chosen).  matmul_forward_splitk_workspace() is a size that never constrains
+ * the choice at GPT-2 shapes.  Calls that overlap on one GPU need a workspace each. */
+#define GPT2HIP_SPLITK_COUNTER_BYTES 16384u
+size_t matmul_forward_splitk_workspace(void);
+int matmul_forward_splitk_status(float* out, const float* inp, const float* weight, const float* bias,
+                                 int B, int T, int C, int OC, int is_gelu, void* workspace,
+                                 size_t workspace_bytes);
+/* The plan matmul_forward_splitk_status would choose: tile shape (0 x 0 for problems outside
+ * the tiled kernels) and workgroups per tile (1 = K not split).  Touches no GPU. */
+int matmul_forward_splitk_plan(int B, int T, int C, int OC, size_t workspace_bytes, int* tile_rows,
+                               int* tile_cols, int* splits);
+/* The same product with the plan given by the caller (tile shape one of those listed at
+ * matmul_forward_tile_shape, 1 <= splits <= C / 32): for parity tests of every kernel form
+ * and for the sweeps that the cost model is fitted to.  Needs C % 32 == 0. */
+int matmul_forward_splitk_forced_status(float* out, const float* inp, const float* weight,
+                                        const float* bias, int B, int T, int C, int OC, int is_gelu,
+                                        void* workspace, size_t workspace_bytes, int tile_rows,
+                                        int tile_cols, int splits);
+
 /* Diagnostic form of matmul_forward (C % 32 == 0, 16-byte aligned operands): the
  * same kernel, which also stores for each of its workgroups four 64-bit words in
  * probe[] (device memory, probe_capacity workgroups): wall clock (100 MHz) at the

@@ -104,3 +104,28 @@ def test_tile_choice_needs_no_gpu_and_avoids_partial_rounds():
             assert rounds * bm * bn <= big * 128 * 192 * 1.45, (M, C, OC, bm, bn)
     with pytest.raises(g2.GPT2HipError):
         g2.matmul_forward_tile_shape(0, 5, 32, 32)
+
+
+def test_splitk_plan_without_a_gpu():
+    """The K-split planner is host arithmetic: no workspace means no split; the BASELINE
+    shapes (exact rounds of the largest tile) never split; fcproj (K = 3072) at short and
+    middling B*T does; every plan fits the workspace it was given."""
+    import importlib
+    g2 = importlib.import_module("cuda-gpt2-inference_amd")
+    ws = g2.lib().matmul_forward_splitk_workspace()
+    assert ws > g2.SPLITK_COUNTER_BYTES
+    for M in (64, 256, 2048, 8192):
+        for C, OC in ((768, 2304), (768, 768), (768, 3072), (3072, 768)):
+            bm, bn, sp = g2.matmul_forward_splitk_plan(1, M, C, OC, 0)
+            assert sp == 1 and (bm, bn) == g2.matmul_forward_tile_shape(1, M, C, OC)
+            bm, bn, sp = g2.matmul_forward_splitk_plan(1, M, C, OC, ws)
+            tiles = -(-M // bm) * -(-OC // bn)
+            assert 1 <= sp <= C // 32
+            assert sp == 1 or tiles * sp * bm * bn * 4 <= ws - g2.SPLITK_COUNTER_BYTES
+            if M == 8192:
+                assert (bm, bn, sp) == (128, 192, 1)
+    for M in (64, 128, 512, 1024, 2048, 3072):
+        assert g2.matmul_forward_splitk_plan(1, M, 3072, 768, ws)[2] > 1, M
+    # a workspace that only holds the counters cannot split
+    assert g2.matmul_forward_splitk_plan(1, 1024, 3072, 768, g2.SPLITK_COUNTER_BYTES)[2] == 1
+    assert g2.matmul_forward_splitk_plan(1, 100, 36, 200, ws) == (0, 0, 1)      # K % 32 != 0

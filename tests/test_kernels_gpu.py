@@ -246,6 +246,83 @@ def test_matmul_every_tile_shape_with_edges(M, C, OC, tile):
     assert_close(out, oracle.matmul_forward(x, w, b), "matmul")
 
 
+# K split between the workgroups of a tile, every kernel form (tile shape x LDS-DMA / ring),
+# ragged edges in both dimensions, split counts that do and do not divide the K slabs.  The
+# same workspace serves all calls: every call must leave its counters at zero.  Two calls
+# give bitwise equal results (the parts are summed in part order whoever arrives last).
+SPLITK_CASES = [
+    (2048, 768, 768, (128, 192), 4), (2045, 3072, 771, (128, 192), 3), (1000, 768, 2300, (128, 128), 2),
+    (1530, 3072, 760, (128, 96), 5), (1024, 768, 768, (64, 128), 8), (1021, 3072, 700, (64, 128), 7),
+    (2048, 768, 2304, (64, 64), 2), (256, 3072, 768, (64, 64), 5), (250, 768, 2300, (64, 64), 3),
+    (256, 3072, 768, (32, 32), 2), (130, 1024, 1000, (32, 32), 4), (64, 96, 50, (32, 32), 3),
+    (2048, 768, 2304, (128, 192), 2),
+]
+
+
+@pytest.fixture(scope="module")
+def splitk_workspace():
+    return g2.matmul_forward_splitk_workspace()
+
+
+@pytest.mark.parametrize("M,C,OC,tile,splits", SPLITK_CASES)
+@pytest.mark.parametrize("gelu", [False, True])
+def test_matmul_splitk_forced(M, C, OC, tile, splits, gelu, splitk_workspace):
+    say(f"matmul split-K M={M} C={C} OC={OC} tile={tile} splits={splits} gelu={gelu}")
+    x, w, b = mm_inputs(M, C, OC, 131)
+    dx, dw, db = dev(x), dev(w), dev(b)
+    outs = []
+    for _ in range(2):
+        full, out, pad = guard((M, OC))
+        g2.matmul_forward_splitk(out, dx, dw, db, 1, M, C, OC, splitk_workspace, is_gelu=gelu,
+                                 plan=(*tile, splits))
+        torch.cuda.synchronize()
+        check_guard(full, pad)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1]), "two runs of a K split differ"
+    assert int(splitk_workspace[:g2.SPLITK_COUNTER_BYTES].max()) == 0, "counters not left at zero"
+    exp = oracle.matmul_forward(x, w, b)
+    if gelu:
+        exp = oracle.gelu_forward(exp)
+    assert_close(outs[0], exp, "matmul split-K")
+
+
+# The plans the cost model picks at the GPT-2 124M shapes over M (with a workspace), against
+# the oracle; at least some of them must split.
+@pytest.mark.parametrize("M", [256, 1024, 2048, 4096])
+def test_matmul_splitk_chosen_plan(M, splitk_workspace):
+    nsplit = 0
+    for C, OC in [(768, 2304), (768, 768), (768, 3072), (3072, 768)]:
+        plan = g2.matmul_forward_splitk_plan(1, M, C, OC, splitk_workspace.numel())
+        say(f"matmul split-K chosen M={M} C={C} OC={OC} plan={plan}")
+        nsplit += plan[2] > 1
+        x, w, b = mm_inputs(M, C, OC, 132)
+        full, out, pad = guard((M, OC))
+        g2.matmul_forward_splitk(out, dev(x), dev(w), dev(b), 1, M, C, OC, splitk_workspace)
+        torch.cuda.synchronize()
+        check_guard(full, pad)
+        assert_close(out, oracle.matmul_forward(x, w, b), "matmul split-K (chosen)")
+    assert int(splitk_workspace[:g2.SPLITK_COUNTER_BYTES].max()) == 0
+    assert M >= 4096 or nsplit > 0
+
+
+def test_matmul_splitk_rejects_what_does_not_fit(splitk_workspace):
+    x, w, b = mm_inputs(64, 64, 64, 133)
+    out = torch.empty((64, 64), device="cuda")
+    with pytest.raises(g2.GPT2HipError):  # 2 K slabs cannot be split three ways
+        g2.matmul_forward_splitk(out, dev(x), dev(w), dev(b), 1, 64, 64, 64, splitk_workspace,
+                                 plan=(32, 32, 3))
+    with pytest.raises(g2.GPT2HipError):  # no such tile
+        g2.matmul_forward_splitk(out, dev(x), dev(w), dev(b), 1, 64, 64, 64, splitk_workspace,
+                                 plan=(48, 48, 2))
+    small = torch.zeros(g2.SPLITK_COUNTER_BYTES + 1024, dtype=torch.uint8, device="cuda")
+    with pytest.raises(g2.GPT2HipError):  # partial tiles do not fit
+        g2.matmul_forward_splitk(out, dev(x), dev(w), dev(b), 1, 64, 64, 64, small, plan=(32, 32, 2))
+    # without a workspace the call is matmul_forward_gelu
+    g2.matmul_forward_splitk(out, dev(x), dev(w), dev(b), 1, 64, 64, 64, None)
+    torch.cuda.synchronize()
+    assert_close(out, oracle.matmul_forward(x, w, b), "matmul split-K without workspace")
+
+
 def test_matmul_lm_head_no_bias():
     # 768 -> 50257 without bias; the oracle runs on a row subset to stay in seconds,
     # which is exact because rows are independent.
