@@ -708,7 +708,14 @@ constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 // accumulators are summed through LDS in a fixed order (ks = 0, 1, ...), so results do
 // not depend on timing.
 // SPLIT: K is also split between `splits` workgroups per tile, as in matmul_dma_kernel.
-template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool GELU, bool SPLIT = false>
+// PIPE: the slab loop is software-pipelined (see below); otherwise a slab is read and
+// multiplied after its barrier.  Measured per shape over B*T = 64 .. 8192: the pipelined loop
+// is 3-11 % faster for 64x96 tiles (whose waves have two k-groups of 12 MFMAs per slab to
+// hide reads under) and up to 35 % SLOWER for 32x32 tiles with few slabs' worth of work per
+// wave, where what counts is how far ahead the fills run: waiting for slab s + 1 before
+// slab s is multiplied costs a slab of lead.
+template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool GELU, bool SPLIT = false,
+          bool PIPE = false>
 __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
     const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn,
@@ -723,7 +730,7 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
   static_assert(BM / 8 % NW == 0 && BN / 8 % NW == 0, "tile/waves mismatch");
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be 32x32 MFMA tiles");
   static_assert(KS == 1 || KS == 2 || KS == 4, "K split must divide the 4 k-groups");
-  static_assert(NBUF >= 2 && (NBUF - 1) * DMA_PER < 64, "vmcnt is a 6-bit counter");
+  static_assert(NBUF >= 2 && NBUF * DMA_PER < 64, "vmcnt is a 6-bit counter");
   constexpr int STAGE_BYTES = (BM + BN) * CHUNKS * 16;
   static_assert((KS - 1) * NMN * TM * TN * 16 * 64 * 4 <= NBUF * STAGE_BYTES,
                 "the K-split reduction reuses the ring's LDS");
@@ -804,33 +811,103 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
     b_addr[i] = (BM * CHUNKS + (wn * WN + (lane & 31)) * CHUNKS + ((2 * g + h) ^ sw)) * 16;
   }
 
-  // Slab s lives in buffer s % NBUF.  Per slab: wait for this wave's fills of slab s,
-  // BARRIER (every wave's fills of slab s have landed and every wave has finished with
-  // slab s-1), refill slab s-1's buffer with slab s+NBUF-1, multiply slab s.
-  int buf = 0;
-  for (int s = 0; s < nslab; s++) {
-    __builtin_amdgcn_s_waitcnt(vmcnt_only((NBUF - 2) * DMA_PER));
-    __syncthreads();
-    dma_slab(s + NBUF - 1, buf == 0 ? NBUF - 1 : buf - 1);
-    const char* const stage = lds_bytes + buf * STAGE_BYTES;
-#pragma unroll
-    for (int g = 0; g < GPW; g++) {
-      f32x4 af[TM], bf[TN];
+  if constexpr (PIPE) {
+    // Slab s lives in buffer s % NBUF; NBUF - 1 fills are in flight behind the slab that is
+    // being multiplied.  Software pipeline, as in matmul_dma_kernel: the operands of a k-group
+    // are read while the MFMAs of the group before it run, and the one barrier per slab sits in
+    // front of the slab's LAST group -- by then every wave has read all of the slab into
+    // registers (its buffer is refilled right away, with slab s + NBUF) and slab s + 1 has
+    // landed for every wave, so that its first operands are read under those last MFMAs.
+    f32x4 af[2][TM], bf[2][TN];
+    auto read_ops = [&](int bufi, int g, int p) {
+      const char* const stage = lds_bytes + bufi * STAGE_BYTES;
 #pragma unroll
       for (int i = 0; i < TM; i++)
-        af[i] = *reinterpret_cast<const f32x4*>(stage + a_addr[g] + i * (32 * BK * 4));
+        af[p][i] = *reinterpret_cast<const f32x4*>(stage + a_addr[g] + i * (32 * BK * 4));
 #pragma unroll
       for (int j = 0; j < TN; j++)
-        bf[j] = *reinterpret_cast<const f32x4*>(stage + b_addr[g] + j * (32 * BK * 4));
+        bf[p][j] = *reinterpret_cast<const f32x4*>(stage + b_addr[g] + j * (32 * BK * 4));
+    };
+    auto mfma_group = [&](int p) {
 #pragma unroll
       for (int e = 0; e < 4; e++)
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
           for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[p][i][e], bf[p][j][e], acc[i][j], 0, 0, 0);
+    };
+#define G2_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+    // one k-group: its TM + TN operand reads each in the shadow of an MFMA, then the other MFMAs
+#define G2_GROUP_SCHEDULE()                                  \
+    _Pragma("unroll") for (int i_ = 0; i_ < TM + TN; i_++) {   \
+      G2_SGB(0x008, 1);                                        \
+      G2_SGB(0x100, 1);                                        \
+    }                                                          \
+    G2_SGB(0x008, 4 * TM * TN - (TM + TN));
+    int buf = 0;
+    auto slab_body = [&](int s, auto parity_tag) {
+      constexpr int P0 = decltype(parity_tag)::value;  // register set holding the slab's first group
+#pragma unroll
+      for (int g = 0; g + 1 < GPW; g++) {
+        read_ops(buf, g + 1, (P0 + g + 1) & 1);
+        mfma_group((P0 + g) & 1);
+        G2_GROUP_SCHEDULE();
+      }
+      __builtin_amdgcn_s_waitcnt(vmcnt_only((NBUF - 2) * DMA_PER));  // my fills of slab s + 1 have landed
+      __syncthreads();
+      dma_slab(s + NBUF, buf);
+      buf = buf + 1 == NBUF ? 0 : buf + 1;
+      read_ops(buf, 0, (P0 + GPW) & 1);
+      mfma_group((P0 + GPW - 1) & 1);
+      G2_GROUP_SCHEDULE();
+    };
+    dma_slab(NBUF - 1, NBUF - 1);  // the NBUF-th fill: every buffer is busy
+    __builtin_amdgcn_s_waitcnt(vmcnt_only((NBUF - 1) * DMA_PER));  // slab 0 has landed
+    __syncthreads();
+    read_ops(0, 0, 0);
+    if constexpr (GPW % 2 == 0) {
+      for (int s = 0; s < nslab; s++) slab_body(s, std::integral_constant<int, 0>{});
+    } else {
+      // an odd number of groups per slab: the register sets swap roles from slab to slab
+      int s = 0;
+      for (; s + 1 < nslab; s += 2) {
+        slab_body(s, std::integral_constant<int, 0>{});
+        slab_body(s + 1, std::integral_constant<int, 1>{});
+      }
+      if (s < nslab) slab_body(s, std::integral_constant<int, 0>{});
     }
-    buf = buf + 1 == NBUF ? 0 : buf + 1;
+#undef G2_GROUP_SCHEDULE
+#undef G2_SGB
+  } else {
+    // Slab s lives in buffer s % NBUF.  Per slab: wait for this wave's fills of slab s,
+    // BARRIER (every wave's fills of slab s have landed and every wave has finished with
+    // slab s-1), refill slab s-1's buffer with slab s+NBUF-1, multiply slab s.
+    int buf = 0;
+    for (int s = 0; s < nslab; s++) {
+      __builtin_amdgcn_s_waitcnt(vmcnt_only((NBUF - 2) * DMA_PER));
+      __syncthreads();
+      dma_slab(s + NBUF - 1, buf == 0 ? NBUF - 1 : buf - 1);
+      const char* const stage = lds_bytes + buf * STAGE_BYTES;
+#pragma unroll
+      for (int g = 0; g < GPW; g++) {
+        f32x4 af[TM], bf[TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+          af[i] = *reinterpret_cast<const f32x4*>(stage + a_addr[g] + i * (32 * BK * 4));
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          bf[j] = *reinterpret_cast<const f32x4*>(stage + b_addr[g] + j * (32 * BK * 4));
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+          for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bf[j][e], acc[i][j], 0, 0, 0);
+      }
+      buf = buf + 1 == NBUF ? 0 : buf + 1;
+    }
   }
   __builtin_amdgcn_s_waitcnt(vmcnt_only(0));  // drain the (unused) fills past the last slab
 
@@ -1210,7 +1287,7 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
 }
 
 // Ring kernel for small problems: K % 32 == 0.
-template <int BM, int BN, int WGM, int WGN, int KS, int NBUF>
+template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool PIPE = false>
 static int launch_ring(float* out, const float* inp, const float* weight, const float* bias, int M,
                        int K, int N, bool gelu, SplitK sk = {}) {
   constexpr int NT = WGM * WGN * KS * kWave;
@@ -1218,11 +1295,11 @@ static int launch_ring(float* out, const float* inp, const float* weight, const 
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
   const long long tiles = (long long)ntm * ntn * sk.splits;
   if (tiles > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
-  auto kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true>
-                  : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false>;
+  auto kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true, false, PIPE>
+                  : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false, false, PIPE>;
   if (sk.splits > 1)
-    kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true, true>
-               : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false, true>;
+    kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true, true, PIPE>
+               : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false, true, PIPE>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
                      K, N, ntm, ntn, sk.ws, sk.cnt, sk.splits);
@@ -1257,12 +1334,13 @@ struct TileCand { int bm, bn; double a, round_us, launch_us, fix_us, fix_part_us
 // (64x192 and 128x64 were fitted too -- a = 1.033 and 1.042 -- and never won by more than
 // 0.4 % anywhere in the sweep: not built)
 static const TileCand kTileCands[] = {
-    {128, 192, 0.988, 6.42, -2.15, 4.21, 0.90, 0.069}, {128, 128, 1.006, 3.59, -0.11, 3.81, 0.64, 0.022},
-    {128, 96, 1.017, 1.84, 1.93, 2.73, 0.54, 0.067},   {64, 128, 1.042, 2.08, 1.01, 2.48, 0.43, 0.0},
-    {64, 64, 1.159, 0.40, 1.88, 1.68, 0.21, 0.116},    {32, 32, 1.398, 0.0, 3.54, 0.90, 0.19, 0.468}};
+    {128, 192, 0.988, 6.42, -2.15, 4.22, 0.90, 0.068}, {128, 128, 1.006, 3.59, -0.11, 3.76, 0.66, 0.020},
+    {128, 96, 1.017, 1.84, 1.93, 2.73, 0.54, 0.066},   {64, 128, 1.042, 2.08, 1.01, 2.30, 0.41, 0.0},
+    {64, 64, 1.159, 0.40, 1.88, 1.65, 0.22, 0.115},    {32, 32, 1.398, 0.0, 3.54, 0.81, 0.20, 0.492},
+    {64, 96, 1.094, 0.98, 3.06, 1.53, 0.44, 0.161}};
 // a split is taken when the model puts it this far ahead of the best plan without one (over
-// the sweep no chosen split is then slower than that plan; 0.9 % behind the best forced plan
-// on average, 5.8 % ahead of the choice without splits)
+// the sweep no chosen split is then slower than that plan; 0.8 % behind the best forced plan
+// on average, 5.1 % ahead of the choice without splits)
 constexpr double kSplitMargin = 1.08;
 constexpr int kTileCandCount = (int)(sizeof(kTileCands) / sizeof(kTileCands[0]));
 constexpr double kCuFlopsPerUs = 579e3;  // what one compute unit sustains in the 128x192 loop
@@ -1335,6 +1413,9 @@ static int launch_choice(int best, long long best_tiles, float* out, const float
                          const float* bias, int M, int C, int OC, bool gelu, unsigned long long* probe,
                          SplitK sk) {
   switch (best) {
+    case 6:
+      // 64x96: two waves side by side, K split between two such pairs
+      return launch_ring<64, 96, 2, 1, 2, 4, true>(out, inp, weight, bias, M, C, OC, gelu, sk);
     case 5:
       // one 32x32 tile per workgroup, its four waves splitting K
       return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu, sk);

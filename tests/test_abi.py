@@ -124,7 +124,7 @@ def test_splitk_plan_without_a_gpu():
             assert sp == 1 or tiles * sp * bm * bn * 4 <= ws - g2.SPLITK_COUNTER_BYTES
             if M == 8192:
                 assert (bm, bn, sp) == (128, 192, 1)
-    for M in (64, 128, 512, 1024, 2048, 3072):
+    for M in (64, 128, 512, 1024, 3072):
         assert g2.matmul_forward_splitk_plan(1, M, 3072, 768, ws)[2] > 1, M
     # a workspace that only holds the counters cannot split
     assert g2.matmul_forward_splitk_plan(1, 1024, 3072, 768, g2.SPLITK_COUNTER_BYTES)[2] == 1
