@@ -54,9 +54,19 @@ constexpr int CHUNKS = BK / 4;   // 16-byte chunks per slab row
 // the 8 XCDs (each with a private L2).  When the number of row tiles divides by
 // 8, XCD x is given the band of row tiles [x*band, (x+1)*band) and walks it
 // column tile by column tile, so that the band's A rows stay in that XCD's L2
-// and each B column tile is fetched once per XCD.
+// and each B column tile is fetched once per XCD.  When the product is wider than
+// it is tall (short prompts: B*T < OC) and the column tiles divide by 8, the bands
+// are bands of column tiles instead: every XCD then reads an eighth of the weights
+// and all of the (smaller) activations, not all of the weights.
+template <int BM, int BN>
 __device__ __forceinline__ void tile_of_block(int pid, int ntm, int ntn, int& tm, int& tn) {
-  if ((ntm & 7) == 0) {
+  if ((ntn & 7) == 0 && (long long)ntn * BN > (long long)ntm * BM) {
+    const int band = ntn >> 3;
+    const int xcd = pid & 7;
+    const int q = pid >> 3;
+    tn = xcd * band + q % band;
+    tm = q / band;
+  } else if ((ntm & 7) == 0) {
     const int band = ntm >> 3;
     const int xcd = pid & 7;
     const int q = pid >> 3;
@@ -194,7 +204,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
   const int wm = wave / WGN, wn = wave % WGN;
 
   int tm, tn;
-  tile_of_block(blockIdx.x, ntm, ntn, tm, tn);
+  tile_of_block<BM, BN>(blockIdx.x, ntm, ntn, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   // ---- global -> register staging --------------------------------------
@@ -453,7 +463,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     pid -= part * (ntm * ntn);
   }
   int tm, tn;
-  tile_of_block(pid, ntm, ntn, tm, tn);
+  tile_of_block<BM, BN>(pid, ntm, ntn, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   // this workgroup's slabs: all of K, or its part of it
   const int slab_lo = SPLIT ? (int)((long long)part * (K / BK) / splits) : 0;
@@ -750,7 +760,7 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
     pid -= part * (ntm * ntn);
   }
   int tm, tn;
-  tile_of_block(pid, ntm, ntn, tm, tn);
+  tile_of_block<BM, BN>(pid, ntm, ntn, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const int slab_lo = SPLIT ? (int)((long long)part * (K / BK) / splits) : 0;
   const int nslab = SPLIT ? (int)((long long)(part + 1) * (K / BK) / splits) - slab_lo : K / BK;
