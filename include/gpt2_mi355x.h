@@ -111,7 +111,9 @@ void matmul_forward_gelu(float* out, const float* inp, const float* weight, cons
  * per-tile counters: zero them once (hipMemset) before the first call; every call leaves them
  * zero.  The rest holds partial tiles (tiles x splits x tile area x 4 bytes; a plan that does
  * not fit is not chosen).  matmul_forward_splitk_workspace() is a size that never constrains
- * the choice at GPT-2 shapes.  Calls that overlap on one GPU need a workspace each. */
+ * the choice at GPT-2 shapes.  Calls that overlap on one GPU need a workspace each.  If a
+ * launch that used the workspace did not run to completion (a device error), zero the
+ * counters again before reusing it. */
 #define GPT2HIP_SPLITK_COUNTER_BYTES 16384u
 size_t matmul_forward_splitk_workspace(void);
 int matmul_forward_splitk_status(float* out, const float* inp, const float* weight, const float* bias,
