@@ -676,6 +676,10 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     return;
   }
   const bool full = (m0 + BM <= M) && (n0 + BN <= N);
+  // A product larger than the 256 MiB Infinity Cache (the logits) will not be read back
+  // from any cache: its tiles are stored with streaming stores, so that they do not push
+  // the operands that other tiles are about to re-read out of L2.
+  const bool stream_out = (size_t)M * N * sizeof(float) > ((size_t)256 << 20);
 #pragma unroll
   for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -683,7 +687,14 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
       const int col = n0 + wn * WN + j * 32 + (lane & 31);
       const int rbase = m0 + wm * WM + i * 32 + 4 * h;
       float* o = out + (size_t)rbase * N + col;
-      if (full) {
+      if (full && stream_out) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          float r = acc[i][j][v];
+          if (GELU) r = gelu_tanh(r);
+          __builtin_nontemporal_store(r, o + (size_t)(8 * (v >> 2) + (v & 3)) * N);
+        }
+      } else if (full) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           float r = acc[i][j][v];
