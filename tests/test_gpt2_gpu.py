@@ -217,6 +217,32 @@ def test_gpt2_graph_replays_match_eager_with_eager_work_between():
         model.close()
 
 
+def test_gpt2_graph_replays_with_k_split_gemms():
+    """A model whose 4C -> C projection splits K between workgroups (C = 256 at B*T = 96): the
+    split's counters are reset by the kernels themselves, so a captured forward must replay to
+    the eager result every time, with eager forwards of another shape in between."""
+    cfg = dict(max_seq_len=64, vocab_size=211, num_layers=2, num_heads=4, channels=256)
+    assert g2.matmul_forward_splitk_plan(2, 48, 1024, 256, g2.lib().matmul_forward_splitk_workspace())[2] > 1
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(syn.make_params(54, perturb_affine=True, **cfg))
+        ids = torch.from_numpy(syn.make_tokens(55, 2, 48, 211)).cuda()
+        other = torch.from_numpy(syn.make_tokens(56, 1, 33, 211)).cuda()
+        model.forward(ids)
+        want = model.logits().clone()
+        exp_logits, _ = oracle.gpt2_forward(syn.make_params(54, perturb_affine=True, **cfg),
+                                            ids.cpu().numpy(), maxT=64, V=211, L=2, NH=4, C=256)
+        assert np.abs(want.cpu().numpy().reshape(exp_logits.shape).astype(np.float64) - exp_logits).max() <= 2e-3
+        for rep in range(4):
+            model.forward_graph(ids)
+            torch.cuda.synchronize()
+            assert torch.equal(model.logits(), want), f"replay {rep}"
+            model.forward(other)
+            torch.cuda.synchronize()
+    finally:
+        model.close()
+
+
 def test_launchers_follow_the_selected_stream():
     cfg = dict(max_seq_len=64, vocab_size=211, num_layers=2, num_heads=2, channels=128)
     model = g2.GPT2(**cfg)
