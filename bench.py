@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 # shapes at M = 8192), from two `rocprofv3 --pmc` runs of `bench.py --pmc-probe`:
 # FETCH_SIZE (scaled x2.0: a 256 MiB copy reads 131 084 KiB on that counter) and
 # WRITE_SIZE (scale 1.0: the same copy writes 262 144 KiB).
-DOMINANT_TRAFFIC_BYTES = int((60717.5 + 21565.5 + 86077.5) / 3 * 2.0 * 1024
+DOMINANT_TRAFFIC_BYTES = int((60798.1 + 21562.0 + 86074.0) / 3 * 2.0 * 1024
                              + (73728 + 24576 + 24576) / 3 * 1024)
 
 
