@@ -654,6 +654,39 @@ __device__ __forceinline__ void lm_head_phase(const DecodeStep& a, float* lds) {
   }
 }
 
+// Workgroups without an attention item would only wait at the phase's barrier.  Instead each
+// reads cache rows on behalf of one item whose workgroup sits in the same XCD (consecutive
+// workgroup ids are dealt round-robin to the 8 XCDs), so that they are in that XCD's L2 when
+// the item asks for them: `first` (this layer's values, which the item wants only after its
+// pass over the keys) and `second` (the next layer's keys, wanted five phases from now).
+// The values are discarded; a wrong guess about the XCD costs nothing but the benefit.
+__device__ __forceinline__ void warm_rows(const DecodeStep& a, const float* first, const float* second, int items) {
+  const int g = (int)blockIdx.x, x = g & 7;
+  const int idle0 = items + ((x - items) & 7);  // the first idle workgroup of this XCD
+  const int item = x + 8 * ((g - idle0) >> 3);  // the XCD's items are x, x + 8, ...
+  // (only while every item finds a helper: with more items than idle workgroups the extra
+  // traffic cost more than the warmed items gained)
+  if (2 * items > (int)gridDim.x || item >= items) return;
+  const size_t base = (size_t)item * a.maxT * 64;
+  const int floats = a.pos * 64;  // rows 0 .. pos-1 of the (sequence, head)
+  f32x4 sink = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int pass = 0; pass < 2; pass++) {
+    const float* rows = pass == 0 ? first : second;
+    if (rows == nullptr) continue;
+    rows += base;
+    for (int i = (int)threadIdx.x * 4; i < floats; i += DS_THREADS * 4 * 8) {
+      f32x4 t[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        t[u] = *reinterpret_cast<const f32x4*>(rows + min(i + u * DS_THREADS * 4, floats - 4));
+#pragma unroll
+      for (int u = 0; u < 8; u++) sink += t[u];
+    }
+  }
+  asm volatile("" : : "v"(sink));
+}
+
 // A step that ends early must not leave the previous step's logits behind as if they were its
 // own: every workgroup that leaves fills the logits it owns in the lm-head phase (the same
 // 16-row groups, for every sequence) with NaN.  Nobody else writes those, so they stay NaN
@@ -716,6 +749,10 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(const DecodeSte
     if ((int)blockIdx.x < items) {
       const int bh = (int)blockIdx.x / a.att_splits;
       attention_item(a, lds, kc, vc, bh / a.NH, bh % a.NH, (int)blockIdx.x % a.att_splits);
+    } else if (a.att_splits == 1) {
+      // this layer's values (the item asks for them only after its pass over the keys) and the
+      // next layer's keys
+      warm_rows(a, vc, l + 1 < a.L ? kc + 2 * a.plane : nullptr, items);
     }
     grid_arrive(a, ++epoch);
     if (!grid_wait(a, lds, epoch)) {
@@ -777,13 +814,16 @@ size_t decode_step_probe_slots(int num_layers) {
 }
 
 // Ranges per (sequence, head) of the attention phase at position pos.  Splitting pays from a
-// few hundred positions on (the projection phase loads S results instead of one: +1.8 us).
-constexpr int kSplitFromPos = 384;
+// few hundred positions on (the projection phase loads S results instead of one: +1.3 us, and
+// with every workgroup holding an item nobody is left to warm cache rows, see warm_rows): from
+// 384 positions where up to four ranges are possible, from 640 where only two are (measured
+// at 5, 6 and 8 sequences: unsplit is ahead up to 600-700 positions, split beyond).
+constexpr int kSplitFromPos = 384, kSplitInTwoFromPos = 640;
 int decode_step_attention_splits(const GPT2Config& c, int B, int pos) {
   if (pos < kSplitFromPos) return 1;
   const int s = DS_GRID / (B * c.num_heads);  // as far as the grid goes
   if (s < 2 || B > 8) return 1;  // the kernel combines ranges only for up to 8 sequences,
-  if (B > 4) return 2;           // and more than 2 of them only for up to 4
+  if (B > 4) return pos < kSplitInTwoFromPos ? 1 : 2;  // and more than 2 of them only for up to 4
   return s > kDecodeMaxSplits ? kDecodeMaxSplits : s;
 }
 

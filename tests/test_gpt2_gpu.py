@@ -320,6 +320,7 @@ def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
     (dict(max_seq_len=400, vocab_size=211, num_layers=2, num_heads=4, channels=256), 1, 380, 8),
     (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=16, channels=1024), 3, 390, 3),
     (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=8, channels=512), 7, 391, 3),
+    (dict(max_seq_len=700, vocab_size=331, num_layers=2, num_heads=8, channels=512), 7, 637, 6),
     (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=8, channels=512), 13, 391, 3),
     # up to the last position the cache holds
     (dict(max_seq_len=1024, vocab_size=211, num_layers=2, num_heads=4, channels=256), 2, 1012, 12),
