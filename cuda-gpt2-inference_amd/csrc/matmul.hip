@@ -2,11 +2,14 @@
 // optional tanh-GELU epilogue.  True fp32 on the matrix cores
 // (v_mfma_f32_32x32x2_f32; gfx950 has no xf32 path).
 //
-// The kernels (the first three share one tiling, LDS layout and MFMA mapping):
+// The kernels (matmul_dma_kernel, matmul_ring_kernel and matmul_mfma_kernel share one tiling,
+// LDS layout and MFMA mapping):
 //   matmul_dma_kernel      K % 32 == 0 (every GPT-2 shape): K slabs go from global
 //                          memory straight into LDS (global_load_lds_dwordx4)
 //   matmul_ring_kernel     the same for problems of few small tiles (short prompts):
 //                          deeper slab ring, optional K split between a tile's waves
+//   (both also in a form that splits K between the workgroups of a tile, for callers that
+//   lend a workspace: splitk_combine, matmul_forward_splitk_status)
 //   matmul_skinny_kernel   at most 16 rows (a decode step): weights streamed through
 //                          registers once, 16x16x4 MFMA, K split over 16 waves
 //   matmul_mfma_kernel     any K % 4 == 0: slabs staged through registers, K tail
