@@ -86,8 +86,9 @@ def test_tile_choice_needs_no_gpu_and_avoids_partial_rounds():
     evenly (128x96: 768 and 256 tiles instead of 384 and 128 tiles of 128x192)."""
     import importlib
     g2 = importlib.import_module("cuda-gpt2-inference_amd")
-    for C, OC in ((768, 2304), (768, 768), (768, 3072), (3072, 768)):
+    for C, OC in ((768, 2304), (768, 768), (3072, 768)):
         assert g2.matmul_forward_tile_shape(8, 1024, C, OC) == (128, 192)
+    assert g2.matmul_forward_tile_shape(8, 1024, 768, 3072) == (256, 192)       # 512 tiles: two exact rounds
     assert g2.matmul_forward_tile_shape(4, 1024, 768, 2304) == (128, 96)
     assert g2.matmul_forward_tile_shape(4, 1024, 768, 768) == (128, 96)
     assert g2.matmul_forward_tile_shape(4, 1024, 1024, 1024) == (128, 128)      # 350M
@@ -123,7 +124,7 @@ def test_splitk_plan_without_a_gpu():
             assert 1 <= sp <= C // 32
             assert sp == 1 or tiles * sp * bm * bn * 4 <= ws - g2.SPLITK_COUNTER_BYTES
             if M == 8192:
-                assert (bm, bn, sp) == (128, 192, 1)
+                assert (bm, bn, sp) == ((256, 192, 1) if OC == 3072 else (128, 192, 1))
     for M in (64, 128, 512, 1024, 3072):
         assert g2.matmul_forward_splitk_plan(1, M, 3072, 768, ws)[2] > 1, M
     # a workspace that only holds the counters cannot split
