@@ -1361,10 +1361,13 @@ static const TileCand kTileCands[] = {
     {128, 192, 0.988, 6.42, -2.15, 4.22, 0.90, 0.068}, {128, 128, 1.006, 3.59, -0.11, 3.76, 0.66, 0.020},
     {128, 96, 1.017, 1.84, 1.93, 2.73, 0.54, 0.066},   {64, 128, 1.042, 2.08, 1.01, 2.30, 0.41, 0.0},
     {64, 64, 1.159, 0.40, 1.88, 1.65, 0.22, 0.115},    {32, 32, 1.398, 0.0, 3.54, 0.81, 0.20, 0.492},
-    {64, 96, 1.094, 0.98, 3.06, 1.53, 0.44, 0.161},    {256, 192, 0.970, 8.5, 4.9, 1e9, 0.0, 0.0}};
+    {64, 96, 1.094, 0.98, 3.06, 1.53, 0.44, 0.161},    {256, 192, 0.970, 7.5, 4.9, 1e9, 0.0, 0.0},
+    {256, 128, 1.000, 2.8, 4.0, 1e9, 0.0, 0.0}};
 // (256x192 -- eight waves of 64x96 -- moves 30 % fewer bytes into LDS per MFMA than 128x192 and
 // wins 1.5-2.5 points where its tiles come out in whole rounds: fc at M = 4096 / 8192, the
-// 350M qkv at 4096 / 8192.  Its K split is never planned: a partial tile is 192 KB.)
+// 350M qkv at 4096 / 8192.  256x128 -- eight waves of 64x64 -- does the same against 128x128 for
+// the 4096-wide fc of the 350M model: 86.7 -> 89.9 % at M = 4096.  Their K split is never
+// planned: a partial tile is 128-192 KB.)
 // a split is taken when the model puts it this far ahead of the best plan without one (over
 // the sweep no chosen split is then slower than that plan; 0.8 % behind the best forced plan
 // on average, 5.1 % ahead of the choice without splits)
@@ -1440,6 +1443,9 @@ static int launch_choice(int best, long long best_tiles, float* out, const float
                          const float* bias, int M, int C, int OC, bool gelu, unsigned long long* probe,
                          SplitK sk) {
   switch (best) {
+    case 8:
+      // eight waves of 64x64, one workgroup per compute unit
+      return launch_dma<256, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
     case 7:
       // eight waves of 64x96, one workgroup per compute unit
       return launch_dma<256, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);

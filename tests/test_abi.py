@@ -89,6 +89,8 @@ def test_tile_choice_needs_no_gpu_and_avoids_partial_rounds():
     for C, OC in ((768, 2304), (768, 768), (3072, 768)):
         assert g2.matmul_forward_tile_shape(8, 1024, C, OC) == (128, 192)
     assert g2.matmul_forward_tile_shape(8, 1024, 768, 3072) == (256, 192)       # 512 tiles: two exact rounds
+    assert g2.matmul_forward_tile_shape(4, 1024, 1024, 4096) == (256, 128)      # 350M fc: 512 tiles
+    assert g2.matmul_forward_tile_shape(4, 1024, 1024, 3072) == (256, 192)      # 350M qkv: 256 tiles
     assert g2.matmul_forward_tile_shape(4, 1024, 768, 2304) == (128, 96)
     assert g2.matmul_forward_tile_shape(4, 1024, 768, 768) == (128, 96)
     assert g2.matmul_forward_tile_shape(4, 1024, 1024, 1024) == (128, 128)      # 350M

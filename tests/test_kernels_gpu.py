@@ -238,7 +238,8 @@ def test_matmul_bias(M, C, OC):
     (3072, 768, 2304, (64, 64)), (3070, 1024, 1000, (64, 64)),
     (1536, 768, 2304, (128, 128)), (4090, 1024, 1020, (128, 128)),
     (2048, 768, 3072, (128, 192)), (500, 768, 768, (32, 32)),
-    (8192, 768, 3072, (256, 192)), (8190, 768, 3070, (256, 192)),
+    (4096, 768, 3072, (256, 192)), (4090, 1024, 3070, (256, 192)),
+    (8190, 768, 3070, (256, 192)), (2040, 1024, 4090, (256, 128)),
 ])
 def test_matmul_every_tile_shape_with_edges(M, C, OC, tile):
     say(f"matmul M={M} C={C} OC={OC} tile={tile}")
@@ -259,7 +260,7 @@ SPLITK_CASES = [
     (256, 3072, 768, (32, 32), 2), (130, 1024, 1000, (32, 32), 4), (64, 96, 50, (32, 32), 3),
     (2048, 768, 2304, (128, 192), 2),
     (2048, 768, 768, (64, 96), 1), (2045, 768, 771, (64, 96), 2), (700, 3072, 2300, (64, 96), 5),
-    (1000, 768, 1000, (256, 192), 1), (500, 1024, 380, (256, 192), 3),
+    (1000, 768, 1000, (256, 192), 1), (500, 1024, 380, (256, 192), 3), (700, 768, 250, (256, 128), 2),
 ]
 
 
