@@ -30,6 +30,7 @@
 // Addresses are buffer addresses (scalar base + scalar row offset + a fixed lane offset):
 // no vector address arithmetic in the loop, and rows at or past T read as zeros.
 //
+#include <algorithm>
 #include <type_traits>
 
 #include "common.hpp"
@@ -602,10 +603,16 @@ int attention_forward_status(float* out, float* qkvr, float* att, const float* i
   if (!out || !inp) return fail(GPT2HIP_EINVAL, "attention_forward: null pointer");
   const int hs = C / NH;
   if (hs == HS && aligned16(inp) && aligned16(out) && (long long)T * 3 * C * 4 < (1LL << 31)) {
-    // two query groups per workgroup, unless that makes fewer than two workgroups per
-    // compute unit (short sequences, few heads): then one group, keys split four ways
+    // Two query groups per workgroup (64 queries, keys split two ways) when there are enough
+    // of them: 768 are resident at once, and a launch is as long as its heaviest workgroup
+    // (T / 64 sub-tiles per wave) unless several rounds of them even that out.  Below that,
+    // one group per workgroup with the keys split four ways: twice the workgroups, each half as
+    // long, at the price of reading every key and value twice as often and a four-way merge.
+    // Measured over T = 384 .. 1024, B = 2 .. 16, 12 and 16 heads, the four-way split wins
+    // (+2 to +19 %) up to about 1.6 T such workgroups, at most 1300, and loses 2-16 % beyond.
     const long long wide = (long long)((T + 63) / 64) * B * NH;
-    const int P = wide < 512 ? 4 : 2;
+    const long long four_way_below = std::max<long long>(512, std::min<long long>(1300, (long long)(1.6 * T)));
+    const int P = wide < four_way_below ? 4 : 2;
     const int bq = 32 * (ATT_WAVES / P);
     const int nqb = (T + bq - 1) / bq;
     const long long blocks = (long long)nqb * B * NH;
