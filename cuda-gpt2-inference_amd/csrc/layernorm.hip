@@ -253,20 +253,32 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   const bool vec = (C % 4 == 0) && C <= 4096 && aligned16(out) && aligned16(inp1) &&
                    aligned16(weight) && aligned16(bias) &&
                    (!FUSED || (aligned16(res_out) && aligned16(inp2)));
-  // several rows per wave once there are enough rows to still fill the chip
+  // Several rows per wave once there are enough rows to still fill the chip.  The fused form,
+  // timed over N = 512 .. 8192 at C = 768 and 1024 (us; rows per wave 1 / 2 / 4 / 8):
+  //   C = 768:  N = 8192: 18.4 / 18.2 / 16.6 / 18.3;  4096: 10.4 / 8.8 / 9.2 / 11.4;
+  //             2048: 5.5 / 5.3 / 7.2 / 9.9;  1024: 3.7 / 4.3 / 6.6 / 9.3
+  //   C = 1024: N = 8192: 24.3 / 23.6 / 22.3 / 21.5;  4096: 14.0 / 11.6 / 12.4 / 14.4;
+  //             2048: 7.5 / 6.4 / 7.6 / 13.4;  1024: 4.9 / 5.0 / 6.8 / 12.3
+  // (eight rows at N = 4096 are 128 workgroups: half the chip idle).
   const bool wide = N >= 4096;
 #define G2_LN(NV, ROWS, EXACT, NTS, ...)                                                        \
   hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED, EXACT, NTS, ##__VA_ARGS__>),       \
                      dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, stream(), \
                      res_out, out, mean, rstd, inp1, inp2, weight, bias, N, C)
 #define G2_LN_ROWS(NV)                                              \
-  if (wide && C == 256 * NV && N % 8 == 0 && (long long)N * C * 4 < (1LL << 31)) { \
+  if (C == 256 * NV && N % 8 == 0 && (long long)N * C * 4 < (1LL << 31) && (FUSED || wide)) { \
     if (!FUSED) {                                                   \
       G2_LN(NV, 2, true, true);                                     \
-    } else if (NV == 4) {                                           \
+    } else if (NV == 4 && N >= 8192) {                              \
       G2_LN(NV, 8, true, false);                                    \
-    } else {                                                        \
+    } else if (N >= 8192) {                                         \
       G2_LN(NV, 4, true, true, FUSED, FUSED);                       \
+    } else if (N >= 2048) {                                         \
+      G2_LN(NV, 2, true, true, FUSED, FUSED);                       \
+    } else if (NV == 4) {                                           \
+      G2_LN(NV, 1, true, false);                                    \
+    } else {                                                        \
+      G2_LN(NV, 1, true, true, FUSED, FUSED);                       \
     }                                                               \
   } else if (wide) {                                                \
     G2_LN(NV, 4, false, false);                                     \

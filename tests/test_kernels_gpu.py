@@ -157,8 +157,12 @@ def test_layernorm_null_stats_and_constant_row():
     assert np.array_equal(out.cpu().numpy(), np.broadcast_to(b, (N, C)))
 
 
+# every form the launcher chooses between by row count: one, two, four and eight rows per wave
+# (N < 2048, < 8192, >= 8192), at 768 and 1024 channels, and the forms with bounds checks
 @pytest.mark.parametrize("N,C", [(8192, 768), (8192, 1024), (256, 768), (5, 64), (7, 260),
-                                 (3, 2048), (9, 4100), (6, 50)])
+                                 (3, 2048), (9, 4100), (6, 50),
+                                 (4096, 768), (4096, 1024), (2048, 1024), (2040, 768), (1000, 1024),
+                                 (1001, 768), (512, 256), (4100, 768), (2048, 2048), (16, 512)])
 def test_fused_residual_layernorm(N, C):
     say(f"fused_residual_layernorm N={N} C={C}")
     x, res, w, b = ln_inputs(N, C, 112)
