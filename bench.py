@@ -374,7 +374,7 @@ def decode_bench(model, cfg, B, T0, steps):
             "lm_head": float((done[5 * L] - passed[5 * L - 1]).mean() / 1e3),
             "work": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in work.items()},
             "barrier": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in wait.items()}}
-    except g2.GPT2HipError:
+    except RuntimeError:  # GPT2HipError: no persistent kernel for this model or batch
         out["persistent_kernel"]["note"] = "the persistent kernel does not take this model or batch"
     log("  decode", json.dumps(out))
     return out

@@ -745,21 +745,22 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
     G2_TRY(skinny_launch(m->step_logits, x, P(P_WTE), nullptr, P(P_LNFW), P(P_LNFB), nullptr, B, C, V,
                          false));
   } else {
-    // More sequences (or sizes the fused kernel does not take): the launchers of the full pass.
+    // More sequences (or sizes the fused kernel does not take): the launchers of the full pass
+    // (beyond 16 sequences the GEMMs are tiled ones and may split K through the workspace).
     G2_TRY(layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, 1, C));
     for (int l = 0; l < L; l++) {
-      G2_TRY(matmul_forward_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs, B,
-                                   1, C, 3 * C));
+      G2_TRY(matmul_forward_splitk_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
+                                          B, 1, C, 3 * C, 0, m->splitk, m->splitk_bytes));
       G2_TRY(attention_decode_launch(m->atty, m->qkv, m->kv + (2 * (size_t)l) * plane,
                                      m->kv + (2 * (size_t)l + 1) * plane, B, pos, c.max_seq_len, C, NH));
-      G2_TRY(matmul_forward_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs, P(P_ATTPROJB) + l * cs,
-                                   B, 1, C, C));
+      G2_TRY(matmul_forward_splitk_status(m->proj, m->atty, P(P_ATTPROJW) + l * cs * cs, P(P_ATTPROJB) + l * cs,
+                                          B, 1, C, C, 0, m->splitk, m->splitk_bytes));
       G2_TRY(fused_residual_layernorm_forward_status(other, m->ln, nullptr, nullptr, residual, m->proj,
                                                      P(P_LN2W) + l * cs, P(P_LN2B) + l * cs, B, 1, C));
-      G2_TRY(matmul_forward_gelu_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs, P(P_FCB) + l * 4 * cs,
-                                        B, 1, C, 4 * C, 1));
-      G2_TRY(matmul_forward_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
-                                   P(P_FCPROJB) + l * cs, B, 1, 4 * C, C));
+      G2_TRY(matmul_forward_splitk_status(m->fch, m->ln, P(P_FCW) + l * 4 * cs * cs, P(P_FCB) + l * 4 * cs,
+                                          B, 1, C, 4 * C, 1, m->splitk, m->splitk_bytes));
+      G2_TRY(matmul_forward_splitk_status(m->proj, m->fch, P(P_FCPROJW) + l * 4 * cs * cs,
+                                          P(P_FCPROJB) + l * cs, B, 1, 4 * C, C, 0, m->splitk, m->splitk_bytes));
       const float* nw = (l + 1 < L) ? P(P_LN1W) + (l + 1) * cs : P(P_LNFW);
       const float* nb = (l + 1 < L) ? P(P_LN1B) + (l + 1) * cs : P(P_LNFB);
       G2_TRY(fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other, m->proj,
