@@ -297,6 +297,10 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
     G2_LN_ROWS(3)
   } else if (C <= 1024) {
     G2_LN_ROWS(4)
+  } else if (C <= 1280) {
+    G2_LN_ROWS(5)  // GPT-2 large
+  } else if (C <= 1792) {
+    G2_LN_ROWS(7)  // GPT-2 XL (1600 channels: 6.25 chunks per lane, the form with bounds checks)
   } else if (C <= 2048) {
     G2_LN_ROWS(8)
   } else {

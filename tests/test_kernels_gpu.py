@@ -162,7 +162,8 @@ def test_layernorm_null_stats_and_constant_row():
 @pytest.mark.parametrize("N,C", [(8192, 768), (8192, 1024), (256, 768), (5, 64), (7, 260),
                                  (3, 2048), (9, 4100), (6, 50),
                                  (4096, 768), (4096, 1024), (2048, 1024), (2040, 768), (1000, 1024),
-                                 (1001, 768), (512, 256), (4100, 768), (2048, 2048), (16, 512)])
+                                 (1001, 768), (512, 256), (4100, 768), (2048, 2048), (16, 512),
+                                 (4096, 1280), (2048, 1600), (300, 1280), (8192, 1600)])
 def test_fused_residual_layernorm(N, C):
     say(f"fused_residual_layernorm N={N} C={C}")
     x, res, w, b = ln_inputs(N, C, 112)
