@@ -40,7 +40,6 @@ namespace g2 {
 constexpr int HS = 64;          // head size this kernel is built for
 constexpr int ATT_THREADS = 256;
 constexpr int ATT_WAVES = ATT_THREADS / kWave;
-constexpr int K_SUB_BYTES = 32 * HS * 4;          // one sub-tile of 32 keys: 8 KiB
 constexpr int WAVE_LDS_BYTES = 34 * kWave * 4;    // a wave's region: its K sub-tile, later its parked partial state
 constexpr float LAZY_LOG2 = 8.0f;  // allowed growth of 2^x above the current shift
 

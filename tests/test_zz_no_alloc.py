@@ -2,7 +2,6 @@
 nothing (its pairs live in a static device array inside the library), called through the C
 ABI and checked bit for bit against matmul_forward_argmax_status, which takes a caller's
 workspace.  Collected last on purpose (file name): a failure here hides no other test."""
-import ctypes
 import importlib
 
 import numpy as np
