@@ -27,12 +27,21 @@ if ROOT not in sys.path:
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense FP32 matrix
 PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
-# HBM bytes per launch of the dominant GEMM kernel (mean of the qkv, attproj and fcproj
-# shapes at M = 8192), from two `rocprofv3 --pmc` runs of `bench.py --pmc-probe`:
-# FETCH_SIZE (scaled x2.0: a 256 MiB copy reads 131 084 KiB on that counter) and
-# WRITE_SIZE (scale 1.0: the same copy writes 262 144 KiB).
-DOMINANT_TRAFFIC_BYTES = int((60798.1 + 21562.0 + 86074.0) / 3 * 2.0 * 1024
-                             + (73728 + 24576 + 24576) / 3 * 1024)
+
+
+def dominant_traffic_bytes():
+    """HBM bytes per launch of the dominant GEMM kernel (mean of the qkv, attproj and fcproj
+    shapes at M = 8192), as recorded in profiles/kernels_baseline_shapes_pmc.txt from two
+    `rocprofv3 --pmc` runs of `bench.py --pmc-probe`: FETCH_SIZE (scaled x2.0: a 256 MiB copy
+    reads 131 101 KiB on that counter) and WRITE_SIZE (scale 1.0).  None if the summary is
+    missing or does not hold the line."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, "profiles", "kernels_baseline_shapes_pmc.txt")).read()
+    except OSError:
+        return None
+    m = re.search(r"dominant kernel of bench\.py.*?:\s*(\d+) bytes of HBM-side traffic per launch", text)
+    return int(m.group(1)) if m else None
 
 
 def log(*a):
@@ -118,6 +127,22 @@ def marker_overhead_ms(g2):
     return us[2] / 1e3
 
 
+def library_ms(g2, fn, **kw):
+    """The same-node vendor-library column of a stand-alone row: `fn` (a torch call, rocBLAS /
+    hipBLASLt / MIOpen / AOTriton underneath) timed with the same events on the same buffers.
+    Outside the product and outside every timed region of the forward pass; a routine that
+    is not available on the box is reported as such."""
+    import torch
+    try:
+        with torch.no_grad():
+            fn(0)
+            torch.cuda.synchronize()
+            return {"library_ms": time_launch(g2, fn, **kw)}
+    except Exception as e:  # noqa: BLE001 - whatever the library raises is the row's note
+        torch.cuda.synchronize()
+        return {"library_ms": None, "library_note": f"unavailable here: {type(e).__name__}: {str(e)[:160]}"}
+
+
 def standalone(g2):
     """Per-kernel figures at the BASELINE shapes (configs 1-3).
 
@@ -126,6 +151,8 @@ def standalone(g2):
     shortest of these kernels runs, which would otherwise be what gets timed.
     """
     import torch
+    import torch.nn.functional as F
+    torch.backends.cuda.matmul.allow_tf32 = False   # the library column is fp32 like ours
     L = g2.lib()
     out = []
     M = 8192
@@ -148,9 +175,17 @@ def standalone(g2):
                          iters=96, warmup=16)
         nbytes = 16 * M * C + 8 * C + 8 * M
         gbs = nbytes / ms / 1e6
-        out.append({"kernel": "fused_residual_layernorm", "shape": f"N={M},C={C}", "ms": ms,
-                    "GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
-                    "note": f"rotating {sets} buffer sets, {sets * 4 * M * C * 4 >> 20} MiB"})
+        row = {"kernel": "fused_residual_layernorm", "shape": f"N={M},C={C}", "ms": ms,
+               "GB/s": gbs, "frac_hbm": gbs / PEAK_HBM_GBS,
+               "note": f"rotating {sets} buffer sets, {sets * 4 * M * C * 4 >> 20} MiB"}
+
+        def torch_ln(i, x=x, r=r, s=s, o=o, w=w, b=b, C=C, sets=sets):
+            k = i % sets
+            torch.add(x[k], r[k], out=s[k])
+            o[k].copy_(F.layer_norm(s[k], (C,), w, b, 1e-5))
+        row.update(library_ms(g2, torch_ln, iters=96, warmup=16))
+        row["library"] = "torch.add + F.layer_norm (+ copy into the output buffer), fp32"
+        out.append(row)
         del x, r, o, s
     # matmul at the GPT-2 124M linear shapes
     for (C, OC, bias) in ((768, 2304, True), (768, 768, True), (768, 3072, True), (3072, 768, True),
@@ -162,8 +197,16 @@ def standalone(g2):
         a = (P(o), P(x), P(w), P(bb) if bias else None, 8, 1024, C, OC)
         ms = time_launch(g2, lambda i: L.matmul_forward(*a), iters=10 if OC > 10000 else 40)
         tf = 2.0 * M * C * OC / ms / 1e9
-        out.append({"kernel": "matmul_forward", "shape": f"M={M},C={C},OC={OC}", "ms": ms,
-                    "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS})
+        row = {"kernel": "matmul_forward", "shape": f"M={M},C={C},OC={OC}", "ms": ms,
+               "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS}
+        lib_fn = ((lambda i: torch.addmm(bb, x, w.t(), out=o)) if bias
+                  else (lambda i: torch.mm(x, w.t(), out=o)))
+        row.update(library_ms(g2, lib_fn, iters=10 if OC > 10000 else 40))
+        row["library"] = ("torch.addmm(bias, x, w^T, out=)" if bias else "torch.mm(x, w^T, out=)") + \
+            " fp32, TF32 off (rocBLAS / hipBLASLt underneath)"
+        if row.get("library_ms"):
+            row["library_frac_fp32_mfma"] = 2.0 * M * C * OC / row["library_ms"] / 1e9 / PEAK_FP32_MFMA_TFLOPS
+        out.append(row)
         del x, w, o
     # K split between workgroups (a lent workspace) where a problem has too few tiles: the
     # 3072 -> 768 projection at B*T below the benchmark's
@@ -193,9 +236,18 @@ def standalone(g2):
         a = (P(o), None, None, P(qkv), B, T, C, NH)
         ms = time_launch(g2, lambda i: L.attention_forward(*a), iters=40)
         tf = 4.0 * B * NH * 64 * T * (T + 1) / 2 / ms / 1e9
-        out.append({"kernel": "attention_forward", "shape": f"B={B},T={T},NH={NH},HS=64", "ms": ms,
-                    "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS})
-        del qkv, o
+        row = {"kernel": "attention_forward", "shape": f"B={B},T={T},NH={NH},HS=64", "ms": ms,
+               "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS}
+        q5 = qkv.view(B, T, 3, NH, 64)
+        qh, kh, vh = (q5[:, :, j].transpose(1, 2) for j in range(3))     # (B, NH, T, 64) views of packed qkv
+        row.update(library_ms(g2, lambda i: F.scaled_dot_product_attention(qh, kh, vh, is_causal=True),
+                              iters=20, warmup=3, groups=3))
+        row["library"] = "torch scaled_dot_product_attention(is_causal=True) fp32 on views of the packed qkv"
+        if row.get("library_ms"):
+            row["library_frac_fp32_mfma"] = (4.0 * B * NH * 64 * T * (T + 1) / 2 / row["library_ms"] / 1e9
+                                            / PEAK_FP32_MFMA_TFLOPS)
+        out.append(row)
+        del qkv, o, q5, qh, kh, vh
     # the other bandwidth kernels at the 124M B=8 T=1024 sizes, rotating buffers
     N = M * 3072
     a4 = torch.randn(4, N, device=dev)
@@ -357,7 +409,10 @@ def decode_bench(model, cfg, B, T0, steps):
         out[name] = {"ms_per_step": ms, "tokens_per_s": B / ms * 1e3, "GB/s": gbs,
                      "frac_hbm": gbs / PEAK_HBM_GBS,
                      "finite": bool(torch.isfinite(model.step_logits()).all())}
-    try:
+    if model.decode_probe_size() == 0:
+        out["persistent_kernel"]["note"] = ("the persistent kernel does not take this model or batch: "
+                                            "both rows are one launch per operation")
+    else:
         # one more step with the persistent kernel's clock probe: per phase kind, the mean time
         # a workgroup works and the mean time from its arrival to everybody's arrival
         clk = model.decode_probe(nxt[0]).cpu().numpy().astype("float64") * 10.0  # ns
@@ -374,8 +429,6 @@ def decode_bench(model, cfg, B, T0, steps):
             "lm_head": float((done[5 * L] - passed[5 * L - 1]).mean() / 1e3),
             "work": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in work.items()},
             "barrier": {n: float(sum(v) / max(len(v), 1) / 1e3) for n, v in wait.items()}}
-    except RuntimeError:  # GPT2HipError: no persistent kernel for this model or batch
-        out["persistent_kernel"]["note"] = "the persistent kernel does not take this model or batch"
     log("  decode", json.dumps(out))
     return out
 
@@ -393,7 +446,8 @@ def cpu_baseline(model, cfg, B, T):
     t0 = time.monotonic()
     oracle.gpt2_forward(params, ids, **kw)
     dt = time.monotonic() - t0
-    return {"value": B * T / dt, "unit": "tokens/s", "cores": oracle.num_threads(), "kind": "port",
+    return {"value": B * T / dt, "unit": "tokens/s", "cores": oracle.num_threads(),
+            "nproc": os.cpu_count(), "cpus_allowed": len(os.sched_getaffinity(0)), "kind": "port",
             "sample": f"one forward of the same workload, B={B}, T={T} ({dt:.2f} s wall); "
                       "plain-C/OpenMP restatement of llm.c's CPU gpt2_forward"}
 
@@ -532,7 +586,7 @@ def main():
     achieved = dom_flops / dom_ms / 1e9
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
                 "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-                "traffic": (DOMINANT_TRAFFIC_BYTES
+                "traffic": (dominant_traffic_bytes()
                             if (args.model == "124M" and B == 8 and T == 1024) else None),
                 "traffic_source": "recorded from two rocprofv3 --pmc runs of bench.py --pmc-probe "
                                   "(profiles/kernels_baseline_shapes_pmc.txt), not counted in this run",

@@ -32,7 +32,7 @@ HIPCC_FLAGS = (
 )
 
 EXPORTS = (
-    "gpt2hip_last_error", "gpt2hip_set_stream", "gpt2hip_get_stream",
+    "gpt2hip_last_error", "gpt2hip_set_stream", "gpt2hip_get_stream", "gpt2hip_set_workspace",
     "encoder_forward", "encoder_forward_status",
     "layernorm_forward", "layernorm_forward_status",
     "fused_residual_layernorm_forward", "fused_residual_layernorm_forward_status",
@@ -172,6 +172,7 @@ def lib() -> ctypes.CDLL:
         L.gpt2_forward_graph_status.restype = ci
         L.gpt2hip_set_stream.argtypes, L.gpt2hip_set_stream.restype = [vp], None
         L.gpt2hip_get_stream.argtypes, L.gpt2hip_get_stream.restype = [], vp
+        L.gpt2hip_set_workspace.argtypes, L.gpt2hip_set_workspace.restype = [vp, cz], ci
         L.gpt2_forward_argmax_status.argtypes = [vp, vp, ci, ci, vp]
         L.gpt2_forward_argmax_status.restype = ci
         L.matmul_forward_argmax_workspace.argtypes = [ci, ci, ci]
@@ -362,6 +363,17 @@ def set_stream(stream) -> None:
     lib().gpt2hip_set_stream(raw or None)
 
 
+def set_workspace(workspace) -> None:
+    """Lend matmul_forward / matmul_forward_gelu of this thread a K-split workspace (a uint8
+    CUDA tensor whose first SPLITK_COUNTER_BYTES were zero before its first use, e.g. from
+    matmul_forward_splitk_workspace(); the caller keeps it alive), or None to take it back."""
+    if workspace is None:
+        _check(lib().gpt2hip_set_workspace(None, 0), "gpt2hip_set_workspace")
+    else:
+        _check(lib().gpt2hip_set_workspace(workspace.data_ptr(), workspace.numel()),
+               "gpt2hip_set_workspace")
+
+
 def read_checkpoint_config(path) -> dict:
     """Header of an llm.c checkpoint file as GPT2(**config) keywords (no GPU needed)."""
     cfg = GPT2Config()
@@ -494,6 +506,10 @@ class GPT2:
                "gpt2_decode_probe")
         phases = 5 * self.config.num_layers + 1
         return clocks.view(phases, 2, -1)
+
+    def decode_probe_size(self) -> int:
+        """Clock slots decode_probe needs; 0 if the next step would not be the persistent kernel."""
+        return int(lib().gpt2_decode_probe_size(self._h))
 
     def decode_options(self, persistent: bool = True, spin_limit: int = 1 << 21):
         """Choose between the persistent decode-step kernel and one launch per operation."""

@@ -28,7 +28,8 @@
 // waves, one barrier per tile, two workgroups per compute unit) ran the benchmark
 // shape B=8, T=1024, NH=12 in 128.8 us where this one takes 121.0 in the same harness.
 // Addresses are buffer addresses (scalar base + scalar row offset + a fixed lane offset):
-// no vector address arithmetic in the loop, and rows at or past T read as zeros.
+// no vector address arithmetic in the loop.  Only a sequence's ragged last sub-tile (T not a
+// multiple of 32) carries its rows in the lane offset, clamped to the sequence's last row.
 //
 #include <algorithm>
 #include <type_traits>
@@ -70,7 +71,9 @@ __device__ __forceinline__ float pair_sum(float x) {
 
 // P = waves that split the keys of one group of 32 queries; a workgroup of 4 waves holds
 // 4 / P such groups.
-template <int P>
+// RAGGED: T is not a multiple of 32, so a sequence's last sub-tile of keys reaches past its
+// rows; that instantiation carries the test for it in its loop, the other one does not.
+template <int P, bool RAGGED>
 __global__ __launch_bounds__(ATT_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ qkv, int T, int NH,
                             int nqb, float scale_log2e) {
@@ -100,8 +103,8 @@ void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ q
   const int diag = qw >> 5;                  // the sub-tile that holds the diagonal; the last one needed
   const bool live = qw < T;                  // a group entirely past T has nothing to do
 
-  // One sequence's packed rows as a buffer: offsets are 32-bit, and rows at or past T read
-  // as zeros (keys there only meet masked or unstored queries).
+  // One sequence's packed rows as a buffer: offsets are 32-bit.  Rows at or past T are never
+  // addressed: the ragged forms below clamp them (keys there only meet masked or unstored queries).
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<float*>(qkv) + (size_t)b * T * 3 * C, 0, T * row_bytes, 0x00020000);
   const int q_col = head * (HS * 4), k_col = q_col + C * 4, v_col = q_col + 2 * C * 4;
@@ -114,12 +117,26 @@ void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ q
   // row & 7 = 4*(i&1) + l/16 for instruction i, so two lane offsets cover all eight.
   const int dma_lane[2] = {(lane >> 4) * row_bytes + (((lane & 15) ^ (lane >> 4)) << 4),
                            (lane >> 4) * row_bytes + (((lane & 15) ^ (4 + (lane >> 4))) << 4)};
+  // The scalar offset of a buffer access is NOT range-checked (only the lane offset is), so a
+  // sub-tile that reaches past T -- the last one of a sequence whose length is not a multiple
+  // of 32 -- takes the form below it: the row goes into the lane offset, clamped to the last
+  // row of the sequence (finite data, and every key there is masked for every stored query).
   auto dma_k = [&](int sub) {
-    const int s0 = sub * 32 * row_bytes + k_col;
+    if (!RAGGED || (sub + 1) * 32 <= T) {
+      const int s0 = sub * 32 * row_bytes + k_col;
 #pragma unroll
-    for (int i = 0; i < 8; i++)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_t*)(my_lds + i * 1024), 16, dma_lane[i & 1],
-                                               s0 + 4 * i * row_bytes, 0, 0);
+      for (int i = 0; i < 8; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_t*)(my_lds + i * 1024), 16, dma_lane[i & 1],
+                                                 s0 + 4 * i * row_bytes, 0, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int row = min(sub * 32 + 4 * i + (lane >> 4), T - 1);
+        const int chunk = ((lane & 15) ^ (4 * (i & 1) + (lane >> 4))) << 4;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_t*)(my_lds + i * 1024), 16,
+                                                 row * row_bytes + chunk, k_col, 0, 0);
+      }
+    }
   };
 
   int sub = part;
@@ -128,8 +145,9 @@ void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ q
   // ---- Q in registers: qreg[g] = Q[myq][8g+4h .. +3] --------------------
   f32x4 qreg[8];
   {
-    const int qv = l32 * row_bytes + h32 * 16;
-    const int qs = qw * row_bytes + q_col;
+    // queries at or past T (RAGGED only; never stored) read the sequence's last row
+    const int qv = (RAGGED ? min(myq, T - 1) : l32) * row_bytes + h32 * 16;
+    const int qs = (RAGGED ? 0 : qw * row_bytes) + q_col;
 #pragma unroll
     for (int g = 0; g < 8; g++)
       qreg[g] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, qv, qs + g * 32, 0));
@@ -166,12 +184,21 @@ void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ q
         kreg[g] = *reinterpret_cast<const f32x4*>(k_addr[g & 3] + (g >> 2) * 128);
       // V of this sub-tile: needed after the scores and the softmax
       f32x2 vreg[16];
-      {
+      if (!RAGGED || k0 + 32 <= T) {
         const int vs = k0 * row_bytes + v_col;
 #pragma unroll
         for (int v = 0; v < 16; v++)
           vreg[v] = __builtin_bit_cast(
               f32x2, __builtin_amdgcn_raw_buffer_load_b64(rsrc, v_lane, vs + (8 * (v >> 2) + (v & 3)) * row_bytes, 0));
+      } else {
+        // the sequence's ragged last sub-tile: rows clamped in the lane offset (see dma_k); the
+        // clamped rows are finite and meet softmax weights that are exactly zero
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int row = min(k0 + 8 * (v >> 2) + (v & 3) + 4 * h32, T - 1);
+          vreg[v] = __builtin_bit_cast(
+              f32x2, __builtin_amdgcn_raw_buffer_load_b64(rsrc, row * row_bytes + l32 * 8, v_col, 0));
+        }
       }
       // the K region is free once its reads have returned: request the next sub-tile
       if (sub + P <= diag) {
@@ -617,12 +644,11 @@ int attention_forward_status(float* out, float* qkvr, float* att, const float* i
     const long long blocks = (long long)nqb * B * NH;
     if (blocks > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "attention_forward: grid too large");
     const float scale_log2e = (1.0f / sqrtf((float)hs)) * 1.4426950408889634f;
-    if (P == 2)
-      hipLaunchKernelGGL(attention_flash_kernel<2>, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out,
-                         inp, T, NH, nqb, scale_log2e);
-    else
-      hipLaunchKernelGGL(attention_flash_kernel<4>, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out,
-                         inp, T, NH, nqb, scale_log2e);
+    const bool ragged = T % 32 != 0;
+    auto kfn = P == 2 ? (ragged ? attention_flash_kernel<2, true> : attention_flash_kernel<2, false>)
+                      : (ragged ? attention_flash_kernel<4, true> : attention_flash_kernel<4, false>);
+    hipLaunchKernelGGL(kfn, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out, inp, T, NH, nqb,
+                       scale_log2e);
   } else {
     if (hs > 256) return fail(GPT2HIP_EINVAL, "attention_forward: head size %d > 256", hs);
     const long long waves = (long long)B * NH * T;

@@ -20,6 +20,14 @@ char* last_error_buffer();  // thread-local, 512 bytes (defined in gpt2.hip)
 hipStream_t& stream_slot();
 inline hipStream_t stream() { return stream_slot(); }
 
+// The K-split workspace that matmul_forward / matmul_forward_gelu of the calling thread use
+// (gpt2hip_set_workspace); none until set.  Defined in gpt2.hip.
+struct ThreadWorkspace {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+ThreadWorkspace& workspace_slot();
+
 inline int fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -180,6 +188,7 @@ struct DecodeStep {
   int att_splits;
   float* logits;              // (B,V)
   unsigned* flags;            // [gridDim.x * FLAG_STRIDE] epochs, then the error word
+  unsigned* error_host;       // pinned host word (device address) that receives the error word too
   unsigned epoch0;            // flags hold values below epoch0 + 1 when the kernel starts
   unsigned spin_limit;
   // optional probe: 100 MHz wall clock of every workgroup g of the G = 256 when it has finished

@@ -104,29 +104,47 @@ __device__ __forceinline__ bool grid_wait(const DecodeStep& a, float* lds, unsig
   int* const bad = reinterpret_cast<int*>(lds + LDS_BAD);
   unsigned* const err = a.flags + (size_t)gridDim.x * FLAG_STRIDE;
   // Wave 0 polls, four flags per lane with all four loads in flight; the other waves come
-  // straight to the barrier below.
+  // straight to the barrier below.  (A poll is a trip to the memory side and back, ~0.9 us, and
+  // a flag that lands just after a poll has passed waits a whole trip for the next one; a second
+  // poll kept in flight half a trip behind the first was measured and is slower, 0.342-0.356
+  // against 0.333 ms per step at 8 sequences: the 256 x 256 flag reads of a poll round are
+  // traffic that the flags themselves have to get through.)
   if (threadIdx.x < kWave) {
     constexpr int PER = DS_GRID / kWave;
     unsigned spins = 0;
-    for (;;) {
-      unsigned v[PER];
+    auto issue = [&](unsigned (&v)[PER]) {
 #pragma unroll
       for (int i = 0; i < PER; i++)
         v[i] = __hip_atomic_load(a.flags + (size_t)(threadIdx.x + kWave * i) * FLAG_STRIDE, __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT);
+    };
+    auto complete = [&](const unsigned (&v)[PER]) {
       bool all = true;
 #pragma unroll
       for (int i = 0; i < PER; i++) all = all && (int)(v[i] - epoch) >= 0;
-      if (all) break;
-      __builtin_amdgcn_s_sleep(2);
+      return all;
+    };
+    // after a poll that did not see everybody: whether to give up (and say so)
+    auto give_up = [&]() {
       ++spins;
       const bool seen = (spins & 63) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (spins > a.spin_limit || seen) {
         // the error word names the step that failed first: position + 1, written once
-        if (!seen) atomicCAS(err, 0u, (unsigned)a.pos + 1u);
+        // (whoever writes it also tells the host, in the pinned word the host looks at once the
+        // step has ended: the host does not copy the device's word behind every step)
+        if (!seen && atomicCAS(err, 0u, (unsigned)a.pos + 1u) == 0u)
+          __hip_atomic_store(a.error_host, (unsigned)a.pos + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         *bad = 1;
-        break;
+        return true;
       }
+      return false;
+    };
+    for (;;) {
+      unsigned v[PER];
+      issue(v);
+      if (complete(v)) break;
+      __builtin_amdgcn_s_sleep(2);
+      if (give_up()) break;
     }
   }
   lds_barrier();
@@ -315,14 +333,17 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
     }
   }
 
+  // The next phase's weights are requested right behind this phase's activations, before
+  // anything waits: loads return in order, so the compiler's own waits for the activations
+  // (a count of the loads issued after them) leave the weights in flight, and these have the
+  // whole phase and its barrier to arrive in.  (Requested only once the activations had arrived,
+  // the last of them were still missing when the phase ended: 0.346 -> 0.337 ms per step at 8
+  // sequences, 0.432 -> 0.420 at 16.)
+  load_next();
   if (LN && 4 * tid < K) {
     *reinterpret_cast<f32x4*>(gb + 4 * tid) = pw.g;
     *reinterpret_cast<f32x4*>(gb + K + 4 * tid) = pw.b;
   }
-  // The activations of this phase have arrived (so has everything requested earlier): the
-  // next phase's weights are requested now and arrive under this phase's arithmetic.
-  wait_vm();
-  load_next();
   if (LN) {
     // Statistics of sequence 4*jg + r4: its row is spread over the 16 blocks of all 4 waves.
     // Two rotations inside each row of 16 lanes sum the row's 4 blocks; the 16 partial sums

@@ -23,6 +23,11 @@ hipStream_t& stream_slot() {
   return s;
 }
 
+ThreadWorkspace& workspace_slot() {
+  static thread_local ThreadWorkspace w;
+  return w;
+}
+
 char* last_error_buffer() {
   static thread_local char buf[512] = {0};
   return buf;
@@ -55,6 +60,7 @@ struct GPT2 {
   size_t pairs_bytes;
   void* splitk;    // workspace of matmul_forward_splitk: counters (zero between calls) + partial tiles
   size_t splitk_bytes;
+  bool splitk_dirty;  // a pass that lent the workspace to its GEMMs did not get to its end
   int last_B, last_T;
   bool last_has_logits;
 
@@ -66,14 +72,15 @@ struct GPT2 {
   int kv_len;    // positions filled so far (the same for every sequence); 0 = empty
 
   // the persistent decode-step kernel: barrier flags + error word on the device, the epoch
-  // its last launch ended with, a pinned host copy of the error word (refreshed after every
-  // step, looked at on the next call)
+  // its last launch ended with, a pinned host word that a step which gives up writes the
+  // error into (looked at on the next call, once the event behind the step has passed)
   unsigned* step_flags;
   float* step_act;  // the activations it hands between workgroups (decode_step_activation_floats)
   unsigned step_epoch;
   unsigned* step_error_host;
-  hipEvent_t step_event;     // recorded behind every copy of the error word to step_error_host
-  bool step_pending;         // a step has been launched whose copy has not been looked at yet
+  unsigned* step_error_device;  // the same pinned word as the device addresses it
+  hipStream_t step_stream;   // the stream of the newest step
+  bool step_pending;         // steps have been launched that nobody has waited for yet
   bool step_fallback;        // a step of the persistent kernel gave up: one launch per operation from then on
   bool step_persistent;      // use the persistent kernel where it takes the model
   unsigned step_spin_limit;  // polls of a barrier flag before a workgroup gives up
@@ -118,11 +125,10 @@ static void free_cache(GPT2* m) {
   if (m->step_act) (void)hipFree(m->step_act);
   m->step_act = nullptr;
   if (m->step_error_host) (void)hipHostFree(m->step_error_host);
-  if (m->step_event) (void)hipEventDestroy(m->step_event);
-  m->step_event = nullptr;
+  m->step_stream = nullptr;
   m->step_pending = false;
   m->kv = m->step_logits = nullptr;
-  m->step_flags = m->step_error_host = nullptr;
+  m->step_flags = m->step_error_host = m->step_error_device = nullptr;
   m->step_epoch = 0;
   m->kv_batch = m->kv_len = 0;
 }
@@ -144,13 +150,22 @@ static int reserve_cache(GPT2* m, int B) {
   if (e == hipSuccess) e = hipMemset(m->step_act, 0, act_bytes);
   if (e == hipSuccess) e = hipHostMalloc((void**)&m->step_error_host, sizeof(unsigned), hipHostMallocDefault);
   if (e == hipSuccess) *m->step_error_host = 0;
-  if (e == hipSuccess) e = hipEventCreateWithFlags(&m->step_event, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipHostGetDevicePointer((void**)&m->step_error_device, m->step_error_host, 0);
   if (e != hipSuccess) {
     free_cache(m);
     return fail(GPT2HIP_ENOMEM, "gpt2: key/value cache for %d sequences (%zu bytes): %s", B, kv_bytes,
                 hipGetErrorString(e));
   }
   m->kv_batch = B;
+  return GPT2HIP_OK;
+}
+
+// The K-split counters are zero between GEMMs that ran to their end.  A pass that returned
+// early (a failed launch) may have left a GEMM in between: the next pass clears them first.
+static int begin_splitk_use(GPT2* m) {
+  if (m->splitk_dirty && m->splitk)
+    G2_HIP(hipMemsetAsync(m->splitk, 0, GPT2HIP_SPLITK_COUNTER_BYTES, stream()));
+  m->splitk_dirty = true;
   return GPT2HIP_OK;
 }
 
@@ -265,6 +280,7 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
     if (rc_step_) return rc_step_;                           \
     if (prof) G2_TRY(prof->mark(cat));                       \
   } while (0)
+  G2_TRY(begin_splitk_use(m));
   if (prof) G2_TRY(prof->mark(-1));
 
   float* residual = m->res_a;  // current residual stream
@@ -304,14 +320,17 @@ static int forward_resident(GPT2* m, int B, int T, Profile* prof = nullptr,
     // rows (b, T-1) of the final layernorm, gathered into the first B rows of m->atty
     G2_HIP(hipMemcpy2DAsync(m->atty, cs * 4, m->ln + (size_t)(T - 1) * cs, (size_t)T * cs * 4, cs * 4, B,
                             hipMemcpyDeviceToDevice, stream()));
-    G2_TRY(matmul_forward_status(m->step_logits, m->atty, P(P_WTE), nullptr, B, 1, C, V));
+    G2_TRY(matmul_forward_splitk_status(m->step_logits, m->atty, P(P_WTE), nullptr, B, 1, C, V, 0, m->splitk,
+                                        m->splitk_bytes));
   } else if (next_ids)
     G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_argmax_status(next_ids, m->pairs, m->pairs_bytes, m->ln,
                                                                   P(P_WTE), nullptr, B, T, C, V));
   else
-    G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_status(m->logits, m->ln, P(P_WTE), nullptr, B, T, C, V));
+    G2_STEP(GPT2_PROF_MATMUL_LMHEAD, matmul_forward_splitk_status(m->logits, m->ln, P(P_WTE), nullptr, B, T, C, V, 0,
+                                                                  m->splitk, m->splitk_bytes));
 #undef G2_STEP
 #undef G2_TRY
+  m->splitk_dirty = false;
   m->last_B = B;
   m->last_T = T;
   m->last_has_logits = next_ids == nullptr && !fill_cache;
@@ -326,6 +345,21 @@ const char* gpt2hip_last_error(void) { return g2::last_error_buffer(); }
 
 void gpt2hip_set_stream(void* hip_stream) { g2::stream_slot() = static_cast<hipStream_t>(hip_stream); }
 void* gpt2hip_get_stream(void) { return g2::stream_slot(); }
+
+int gpt2hip_set_workspace(void* workspace, size_t workspace_bytes) {
+  using namespace g2;
+  if (!workspace || workspace_bytes == 0) {
+    workspace_slot() = ThreadWorkspace{};
+    return GPT2HIP_OK;
+  }
+  if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+    return fail(GPT2HIP_EINVAL, "gpt2hip_set_workspace: workspace must be 256-byte aligned");
+  if (workspace_bytes < GPT2HIP_SPLITK_COUNTER_BYTES)
+    return fail(GPT2HIP_EINVAL, "gpt2hip_set_workspace: %zu bytes do not hold the %u bytes of counters",
+                workspace_bytes, GPT2HIP_SPLITK_COUNTER_BYTES);
+  workspace_slot() = ThreadWorkspace{workspace, workspace_bytes};
+  return GPT2HIP_OK;
+}
 
 GPT2* gpt2_create(const GPT2Config* config) {
   using namespace g2;
@@ -571,18 +605,17 @@ namespace g2 {
 // operation from then on.  Returns an error exactly once per failure.
 static int settle_steps(GPT2* m, bool wait) {
   if (!m->step_pending) return GPT2HIP_OK;
+  // The workgroup that gives up writes the pinned word itself (system scope), so a look at it
+  // costs nothing and needs no event behind every step; only a caller that wants to be sure that
+  // every queued step has ended waits, for the stream the steps were queued on.
   if (wait) {
-    G2_HIP(hipEventSynchronize(m->step_event));
-  } else {
-    const hipError_t q = hipEventQuery(m->step_event);
-    if (q == hipErrorNotReady) return GPT2HIP_OK;
-    G2_HIP(q);
+    G2_HIP(hipStreamSynchronize(m->step_stream));
+    m->step_pending = false;
   }
-  m->step_pending = false;
-  const unsigned word = *m->step_error_host;
+  const unsigned word = __atomic_load_n(m->step_error_host, __ATOMIC_ACQUIRE);
   if (word == 0) return GPT2HIP_OK;
   *m->step_error_host = 0;
-  G2_HIP(hipMemsetAsync(m->step_flags, 0, decode_step_flag_bytes(m->device), stream()));
+  G2_HIP(hipMemsetAsync(m->step_flags, 0, decode_step_flag_bytes(m->device), m->step_stream));
   m->step_epoch = 0;
   m->step_fallback = true;
   const int failed = (int)word - 1;
@@ -604,7 +637,7 @@ int gpt2_prefill_status(GPT2* model, const int* inputs_device, int B, int T) {
   if (!model) return fail(GPT2HIP_EINVAL, "gpt2_prefill: null model");
   // a failure among earlier decode steps that nobody has asked about: the cache is rebuilt
   // here anyway, so only the recovery (cleared barrier state, launch-per-operation steps) matters
-  (void)settle_steps(model, true);
+  if (settle_steps(model, true)) last_error_buffer()[0] = 0;  // not this call's failure
   if (int rc = reserve(model, B, T)) return rc;
   if (!inputs_device) return fail(GPT2HIP_EINVAL, "gpt2_prefill: null inputs");
   if (model->kv_batch != B) {  // the cache planes are indexed with the batch it was sized for
@@ -670,12 +703,10 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
   // are reused.
   float* residual = m->res_a;
   float* other = m->res_b;
-  G2_HIP(hipMemcpyAsync(m->ids, next_ids_device, (size_t)B * sizeof(int), hipMemcpyDeviceToDevice,
-                        stream()));
   const bool persistent = m->step_persistent && !m->step_fallback && m->step_flags && m->step_act &&
                           decode_step_supported(c, B, m->device);
-  if (!persistent)  // the persistent kernel gathers the embeddings itself
-    G2_TRY(encoder_launch(residual, m->ids, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
+  if (!persistent)  // the persistent kernel gathers the embeddings itself, from the caller's ids
+    G2_TRY(encoder_launch(residual, next_ids_device, P(P_WTE), P(P_WPE) + (size_t)pos * cs, B, 1, C, V));
   const size_t plane = (size_t)m->kv_batch * c.max_seq_len * cs;
   if (persistent) {
     // one persistent kernel for the whole step
@@ -696,7 +727,7 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
     st.fcprojb = P(P_FCPROJB);
     st.lnfw = P(P_LNFW);
     st.lnfb = P(P_LNFB);
-    st.ids = m->ids;
+    st.ids = next_ids_device;  // read in stream order, like a copy of them would be
     st.kv = m->kv;
     st.plane = plane;
     st.x = m->step_act;
@@ -718,12 +749,11 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
     st.V = V;
     st.pos = pos;
     st.maxT = c.max_seq_len;
+    st.error_host = m->step_error_device;
     G2_TRY(decode_step_launch(st, c, m->device));
     m->step_epoch += 5u * (unsigned)L + 8u;
-    G2_HIP(hipMemcpyAsync(m->step_error_host, (const char*)m->step_flags + decode_step_flag_bytes(m->device) -
-                                                  16 * sizeof(unsigned),
-                          sizeof(unsigned), hipMemcpyDeviceToHost, stream()));
-    G2_HIP(hipEventRecord(m->step_event, stream()));
+    // (no copy of the error word: the workgroup that gives up writes it to the pinned host word itself)
+    m->step_stream = stream();
     m->step_pending = true;
   } else if (skinny_supported(B, C, true, residual, m->params) && skinny_supported(B, 4 * C, false, m->fch, m->params)) {
     // Up to 16 sequences: five launches per block.  The layernorms run inside the GEMMs
@@ -747,6 +777,7 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
   } else {
     // More sequences (or sizes the fused kernel does not take): the launchers of the full pass
     // (beyond 16 sequences the GEMMs are tiled ones and may split K through the workspace).
+    G2_TRY(begin_splitk_use(m));
     G2_TRY(layernorm_forward_status(m->ln, nullptr, nullptr, residual, P(P_LN1W), P(P_LN1B), B, 1, C));
     for (int l = 0; l < L; l++) {
       G2_TRY(matmul_forward_splitk_status(m->qkv, m->ln, P(P_QKVW) + l * 3 * cs * cs, P(P_QKVB) + l * 3 * cs,
@@ -766,7 +797,9 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
       G2_TRY(fused_residual_layernorm_forward_status(residual, m->ln, nullptr, nullptr, other, m->proj,
                                                      nw, nb, B, 1, C));
     }
-    G2_TRY(matmul_forward_status(m->step_logits, m->ln, P(P_WTE), nullptr, B, 1, C, V));
+    G2_TRY(matmul_forward_splitk_status(m->step_logits, m->ln, P(P_WTE), nullptr, B, 1, C, V, 0, m->splitk,
+                                        m->splitk_bytes));
+    m->splitk_dirty = false;
   }
 #undef G2_TRY
   m->kv_len = pos + 1;
@@ -777,10 +810,14 @@ static int decode_step(GPT2* model, const int* next_ids_device, unsigned long lo
 
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit) {
   if (!model) return g2::fail(GPT2HIP_EINVAL, "gpt2_decode_options: null model");
+  // A failed step nobody has asked about yet is settled first (cache rolled back, barrier state
+  // cleared): settling it later would switch the persistent kernel off again behind this
+  // call's back.  Its failure is still reported, by this call's return value.
+  const int pending = g2::settle_steps(model, true);
   if (persistent != 0) model->step_fallback = false;  // asked for (again) explicitly
   model->step_persistent = persistent != 0;
   model->step_spin_limit = spin_limit;
-  return GPT2HIP_OK;
+  return pending;
 }
 
 const float* gpt2_step_logits(const GPT2* model) { return model ? model->step_logits : nullptr; }
@@ -805,6 +842,13 @@ int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, i
     return fail(GPT2HIP_EINVAL, "gpt2_forward_profiled: null pointer");
   G2_HIP(hipMemcpyAsync(model->ids, inputs_device, (size_t)B * T * sizeof(int),
                         hipMemcpyDeviceToDevice, stream()));
+  // The pass's first launch, issued once untimed (it is idempotent): the opening event then
+  // sits between two back-to-back launches like every other event of the pass, instead of
+  // behind the copy of the ids and the device's wake-up from idle.
+  if (int rc = encoder_launch(model->res_a, model->ids, model->params + model->param_off[P_WTE],
+                              model->params + model->param_off[P_WPE], B, T, model->cfg.channels,
+                              model->cfg.vocab_size))
+    return rc;
   Profile prof;
   if (int rc = forward_resident(model, B, T, &prof)) return rc;
   G2_HIP(hipEventSynchronize(prof.events.back()));

@@ -45,6 +45,7 @@
 #include <algorithm>
 #include <mutex>
 #include <type_traits>
+#include <unordered_set>
 
 #include "common.hpp"
 
@@ -1219,18 +1220,16 @@ __global__ __launch_bounds__(256) void matmul_argmax_generic_kernel(int* __restr
 // Raises the dynamic-LDS limit of a kernel, once per (thread, device, kernel).
 static int allow_lds(const void* kfn, size_t lds_bytes) {
   static thread_local int configured_for = -1;
-  static thread_local const void* configured[64];
-  static thread_local int nconfigured = 0;
+  static thread_local std::unordered_set<const void*> configured;  // grows with the forms touched
   int dev = 0;
   G2_HIP(hipGetDevice(&dev));
   if (configured_for != dev) {
     configured_for = dev;
-    nconfigured = 0;
+    configured.clear();
   }
-  for (int i = 0; i < nconfigured; i++)
-    if (configured[i] == kfn) return GPT2HIP_OK;
+  if (configured.count(kfn)) return GPT2HIP_OK;
   G2_HIP(hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  if (nconfigured < 64) configured[nconfigured++] = kfn;
+  configured.insert(kfn);
   return GPT2HIP_OK;
 }
 
@@ -1602,7 +1601,8 @@ extern "C" {
 
 int matmul_forward_status(float* out, const float* inp, const float* weight, const float* bias,
                           int B, int T, int C, int OC) {
-  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false);
+  const g2::ThreadWorkspace& w = g2::workspace_slot();  // gpt2hip_set_workspace; none by default
+  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false, nullptr, nullptr, w.ptr, w.bytes);
 }
 
 void matmul_forward(float* out, const float* inp, const float* weight, const float* bias, int B,
@@ -1705,7 +1705,9 @@ int matmul_forward_splitk_plan(int B, int T, int C, int OC, size_t workspace_byt
 
 int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,
                                const float* bias, int B, int T, int C, int OC, int is_gelu) {
-  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, is_gelu != 0);
+  const g2::ThreadWorkspace& w = g2::workspace_slot();
+  return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, is_gelu != 0, nullptr, nullptr, w.ptr,
+                             w.bytes);
 }
 
 void matmul_forward_gelu(float* out, const float* inp, const float* weight, const float* bias,

@@ -88,31 +88,29 @@ int main(int argc, char** argv) {
   HIP_OK(hipMalloc((void**)&mean, M * 4));
   HIP_OK(hipMalloc((void**)&rstd, M * 4));
   HIP_OK(hipMemcpy(ids, hids.data(), M * sizeof(int), hipMemcpyHostToDevice));
-  // A caller that owns its buffers can lend the GEMMs a workspace (counters zeroed once), with
-  // which a layer of few tiles splits K between workgroups; the library's own driver does, so
-  // this one does too.  matmul_forward / matmul_forward_gelu are the same calls without it.
+  // llm.c's launcher signatures have no argument for a workspace.  A caller that owns its buffers
+  // lends the GEMMs one through the calling thread's setting instead (counters zeroed once): with
+  // it matmul_forward / matmul_forward_gelu split K between workgroups where a layer has few
+  // tiles, exactly as the library's own driver does with the workspace its model owns.
   void* ws;
   const size_t ws_bytes = matmul_forward_splitk_workspace();
   HIP_OK(hipMalloc(&ws, ws_bytes));
   HIP_OK(hipMemset(ws, 0, GPT2HIP_SPLITK_COUNTER_BYTES));
-  auto matmul_ws = [&](float* out, const float* inp, const float* weight, const float* bias, int OC_in,
-                       int OC_out, int is_gelu) {
-    if (matmul_forward_splitk_status(out, inp, weight, bias, B, T, OC_in, OC_out, is_gelu, ws, ws_bytes)) {
-      fprintf(stderr, "matmul_forward_splitk_status: %s\n", gpt2hip_last_error());
-      exit(2);
-    }
-  };
+  if (gpt2hip_set_workspace(ws, ws_bytes) != GPT2HIP_OK) {
+    fprintf(stderr, "gpt2hip_set_workspace: %s\n", gpt2hip_last_error());
+    return 2;
+  }
 
   float *residual = res_a, *other = res_b;
   encoder_forward(residual, ids, wte, wpe, B, T, C);
   layernorm_forward(ln, mean, rstd, residual, ln1w, ln1b, B, T, C);
   for (int l = 0; l < L; l++) {
-    matmul_ws(qkv, ln, qkvw + l * 3 * c * c, qkvb + l * 3 * c, C, 3 * C, 0);
+    matmul_forward(qkv, ln, qkvw + l * 3 * c * c, qkvb + l * 3 * c, B, T, C, 3 * C);
     attention_forward(atty, /*qkvr=*/nullptr, /*att=*/nullptr, qkv, B, T, C, NH);
-    matmul_ws(proj, atty, attprojw + l * c * c, attprojb + l * c, C, C, 0);
+    matmul_forward(proj, atty, attprojw + l * c * c, attprojb + l * c, B, T, C, C);
     fused_residual_layernorm_forward(other, ln, mean, rstd, residual, proj, ln2w + l * c, ln2b + l * c, B, T, C);
-    matmul_ws(fch, ln, fcw + l * 4 * c * c, fcb + l * 4 * c, C, 4 * C, /*is_gelu=*/1);
-    matmul_ws(proj, fch, fcprojw + l * 4 * c * c, fcprojb + l * c, 4 * C, C, 0);
+    matmul_forward_gelu(fch, ln, fcw + l * 4 * c * c, fcb + l * 4 * c, B, T, C, 4 * C, /*is_gelu=*/1);
+    matmul_forward(proj, fch, fcprojw + l * 4 * c * c, fcprojb + l * c, B, T, 4 * C, C);
     const float* nw = (l + 1 < L) ? ln1w + (l + 1) * c : lnfw;
     const float* nb = (l + 1 < L) ? ln1b + (l + 1) * c : lnfb;
     fused_residual_layernorm_forward(residual, ln, mean, rstd, other, proj, nw, nb, B, T, C);
@@ -149,6 +147,7 @@ int main(int argc, char** argv) {
          "finite=%d status_form_reports=%d\n", L, C, B, T, V, sum, maxdiff, (int)finite, (int)reports);
 
   gpt2_destroy(model);
+  gpt2hip_set_workspace(nullptr, 0);
   void* bufs[] = {params, ids, res_a, res_b, ln, qkv, atty, proj, fch, logits, mean, rstd, ws};
   for (void* p : bufs) HIP_OK(hipFree(p));
   return (finite && maxdiff == 0.0 && reports) ? 0 : 1;

@@ -274,7 +274,9 @@ int gpt2_decode_status(GPT2* model, const int* next_ids_device);
  * rolled back to the positions before the failed step (gpt2_cache_length()), so decoding can
  * resume from there, and the model runs one launch per operation until gpt2_decode_options
  * asks for the persistent kernel again.  gpt2_prefill_status clears a failure nobody asked
- * about (it rebuilds the cache anyway). */
+ * about (it rebuilds the cache anyway).  gpt2_decode_options itself waits for the steps queued
+ * so far and, if one of them gave up and nobody has been told yet, applies the new options and
+ * then returns that failure (rolled-back cache as above) instead of 0. */
 int gpt2_decode_options(GPT2* model, int persistent, unsigned spin_limit);
 /* Waits until every decode step queued so far has ended and reports whether one of the
  * persistent kernel's steps gave up (see gpt2_decode_options); 0 if all of them completed.
@@ -333,6 +335,20 @@ int gpt2_argmax_status(GPT2* model, int* ids_device);
  * on the null stream throughout (train_gpt2_fp32.cu), which is therefore the default. */
 void gpt2hip_set_stream(void* hip_stream);
 void* gpt2hip_get_stream(void);
+
+/* A K-split workspace for the launchers that keep llm.c's signatures.  matmul_forward(out,
+ * inp, weight, bias, B, T, C, OC) (reference kernels/matmul/2_matmul_cublas.cuh:34-42) and
+ * matmul_forward_gelu (kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:237-246) have no
+ * argument through which a caller could lend one; a caller that sets one here gets, from
+ * those two launchers on the calling thread, exactly what matmul_forward_splitk_status gives
+ * with the same workspace (same plan, same bits).  Same contract as there: device memory,
+ * 256-byte aligned, the first GPT2HIP_SPLITK_COUNTER_BYTES zeroed once before the first use,
+ * and ONE workspace per set of launches that may overlap on the GPU -- two threads, or two
+ * streams of one thread, must not share one.  NULL / 0, the initial value, means none: the
+ * launchers then choose a tile shape only.  The library's own gpt2_forward driver uses a
+ * workspace that the model owns and ignores this setting.  Returns GPT2HIP_EINVAL for a
+ * misaligned pointer or a size below the counters'. */
+int gpt2hip_set_workspace(void* workspace, size_t workspace_bytes);
 
 /* Event timer on the calling thread's stream (the stream its launchers use). */
 typedef struct GPT2Timer GPT2Timer;

@@ -132,3 +132,27 @@ def test_splitk_plan_without_a_gpu():
     # a workspace that only holds the counters cannot split
     assert g2.matmul_forward_splitk_plan(1, 1024, 3072, 768, g2.SPLITK_COUNTER_BYTES)[2] == 1
     assert g2.matmul_forward_splitk_plan(1, 100, 36, 200, ws) == (0, 0, 1)      # K % 32 != 0
+
+
+def test_thread_workspace_setting_is_validated_without_a_gpu():
+    """gpt2hip_set_workspace only records a pointer: alignment and size are checked up front."""
+    L = g2.lib()
+    assert L.gpt2hip_set_workspace(ctypes.c_void_p(4096 + 64), 1 << 20) == 1
+    assert b"aligned" in L.gpt2hip_last_error()
+    assert L.gpt2hip_set_workspace(ctypes.c_void_p(4096), 1024) == 1
+    assert b"counters" in L.gpt2hip_last_error()
+    assert L.gpt2hip_set_workspace(ctypes.c_void_p(4096), 1 << 20) == 0
+    assert L.gpt2hip_set_workspace(None, 0) == 0
+
+
+def test_library_links_no_blas():
+    """The product is hand-written HIP: the shared library must not depend on a vendor BLAS
+    (rocBLAS / hipBLAS / hipBLASLt), not even indirectly through its own link line."""
+    import subprocess
+    out = subprocess.run(["readelf", "-d", g2.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    needed = re.findall(r"\(NEEDED\)\s+Shared library: \[(.*?)\]", out)
+    assert needed, out
+    assert not [n for n in needed if re.search(r"blas|miopen|rccl|torch", n, re.I)], needed
+    syms = subprocess.run(["nm", "-D", "--undefined-only", g2.LIB_PATH], capture_output=True, text=True,
+                          check=True).stdout
+    assert not re.search(r"rocblas_|hipblas|hipblaslt", syms, re.I)

@@ -324,6 +324,12 @@ def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
     (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=8, channels=512), 13, 391, 3),
     # up to the last position the cache holds
     (dict(max_seq_len=1024, vocab_size=211, num_layers=2, num_heads=4, channels=256), 2, 1012, 12),
+    # five and nine sequences (two and three groups of four per phase) at the widest model, and
+    # batches beyond the persistent kernel's sixteen, which take one launch per operation
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=4, channels=256), 5, 21, 3),
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=16, channels=1024), 9, 30, 3),
+    (dict(max_seq_len=48, vocab_size=1031, num_layers=2, num_heads=12, channels=768), 17, 20, 3),
+    (dict(max_seq_len=48, vocab_size=331, num_layers=2, num_heads=12, channels=768), 64, 30, 3),
 ])
 def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_path(cfg, B, T0, steps):
     print(f"persistent decode cfg={cfg} B={B} T0={T0} steps={steps}", flush=True)
@@ -340,6 +346,8 @@ def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_
         for persistent in (False, True):
             model.decode_options(persistent=persistent)
             model.prefill(dids[:, :T0].contiguous())
+            # the path that is meant runs: the persistent kernel takes up to 16 sequences
+            assert (model.decode_probe_size() > 0) == (persistent and B <= 16)
             out = []
             for s in range(steps):
                 print(f"  persistent={persistent} step {s}", flush=True)
@@ -429,14 +437,29 @@ def test_gpt2_persistent_decode_gives_up_a_barrier_wait_cleanly():
         got = model.decode(ids[:, 7].contiguous())
         model.decode_sync()
         assert (got - want7).abs().max().item() <= 1e-4
-        # a failure nobody asked about does not outlive the next prompt
+        assert g2.lib().gpt2_decode_probe_size(model._h) > 0      # ... and it is the persistent kernel
+        # a failure nobody asked about does not outlive the next prompt, and the prompt's own
+        # call succeeds without a stale message
         model.decode_options(persistent=True, spin_limit=0)
         model.decode(ids[:, 8].contiguous())
-        model.decode_options(persistent=True)
         model.prefill(ids[:, :7].contiguous())
+        assert g2.lib().gpt2hip_last_error() == b""
+        model.decode_options(persistent=True)
+        assert g2.lib().gpt2_decode_probe_size(model._h) > 0
         got = model.decode(ids[:, 7].contiguous())
         model.decode_sync()
         assert (got - want7).abs().max().item() <= 1e-4
+        # gpt2_decode_options settles a failure that is still pending (and reports it) before it
+        # re-enables the persistent kernel, so that the request is not undone behind its back
+        model.decode_options(persistent=True, spin_limit=0)
+        model.decode(ids[:, 8].contiguous())
+        with pytest.raises(g2.GPT2HipError, match="grid barrier"):
+            model.decode_options(persistent=True)
+        assert model.cache_length() == 8
+        assert g2.lib().gpt2_decode_probe_size(model._h) > 0      # the options were applied all the same
+        got8b = model.decode(ids[:, 8].contiguous())
+        model.decode_sync()
+        assert (got8b - want8).abs().max().item() <= 1e-4
     finally:
         model.close()
 

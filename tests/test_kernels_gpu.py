@@ -315,6 +315,41 @@ def test_matmul_splitk_chosen_plan(M, splitk_workspace):
     assert nsplit > 0
 
 
+@pytest.mark.parametrize("M", [256, 1024, 3072])
+def test_matmul_llmc_signature_splits_k_through_the_thread_workspace(M, splitk_workspace):
+    """matmul_forward / matmul_forward_gelu carry no workspace argument; with one lent through
+    gpt2hip_set_workspace they give matmul_forward_splitk's result bit for bit (the same plan),
+    and with none they are as before."""
+    C, OC = 3072, 768
+    plan = g2.matmul_forward_splitk_plan(1, M, C, OC, splitk_workspace.numel())
+    say(f"matmul_forward with a thread workspace M={M} C={C} OC={OC} plan={plan}")
+    assert plan[2] > 1
+    x, w, b = mm_inputs(M, C, OC, 134)
+    dx, dw, db = dev(x), dev(w), dev(b)
+    want = torch.empty((M, OC), device="cuda")
+    g2.matmul_forward_splitk(want, dx, dw, db, 1, M, C, OC, splitk_workspace)
+    want_gelu = torch.empty((M, OC), device="cuda")
+    g2.matmul_forward_splitk(want_gelu, dx, dw, db, 1, M, C, OC, splitk_workspace, is_gelu=True)
+    plain = torch.empty((M, OC), device="cuda")
+    g2.matmul_forward(plain, dx, dw, db, 1, M, C, OC)
+    g2.set_workspace(splitk_workspace)
+    try:
+        full, out, pad = guard((M, OC))
+        g2.matmul_forward(out, dx, dw, db, 1, M, C, OC)
+        out_gelu = torch.empty((M, OC), device="cuda")
+        g2.matmul_forward_gelu(out_gelu, dx, dw, db, 1, M, C, OC, True)
+        torch.cuda.synchronize()
+        check_guard(full, pad)
+        assert torch.equal(out, want) and torch.equal(out_gelu, want_gelu)
+        assert_close(out, oracle.matmul_forward(x, w, b), "matmul_forward (thread workspace)")
+        assert int(splitk_workspace[:g2.SPLITK_COUNTER_BYTES].max()) == 0
+    finally:
+        g2.set_workspace(None)
+    again = torch.empty((M, OC), device="cuda")
+    g2.matmul_forward(again, dx, dw, db, 1, M, C, OC)
+    assert torch.equal(again, plain)
+
+
 def test_matmul_splitk_rejects_what_does_not_fit(splitk_workspace):
     x, w, b = mm_inputs(64, 64, 64, 133)
     out = torch.empty((64, 64), device="cuda")
@@ -439,6 +474,28 @@ def test_attention_hs64(B, T, NH):
     check_guard(full, pad)
     assert np.array_equal(dq.cpu().numpy(), qkv), "attention must not write its input"
     assert_close(out, oracle.attention_forward(qkv, NH), "attention")
+
+
+@pytest.mark.parametrize("B,T,NH", [(2, 33, 3), (1, 130, 2), (3, 95, 1), (2, 1, 2)])
+def test_attention_ragged_length_never_reads_past_its_rows(B, T, NH):
+    """T is not a multiple of the 32-key sub-tile: the rows behind the last sequence must not
+    reach the result.  qkv is a view into a larger tensor whose other elements are NaN (so
+    nothing is read outside an allocation); a value row past T that met a zero softmax weight
+    would still turn the whole query group into NaN."""
+    say(f"attention ragged B={B} T={T} NH={NH} inside NaN")
+    C = NH * 64
+    qkv = np.random.default_rng(134).standard_normal((B, T, 3 * C), dtype=np.float32)
+    n = qkv.size
+    pad = 64 * 3 * C  # two sub-tiles' worth of rows on either side
+    big = torch.full((n + 2 * pad,), float("nan"), device="cuda")
+    big[pad:pad + n] = dev(qkv).view(-1)
+    dq = big[pad:pad + n].view(B, T, 3 * C)
+    full, out, opad = guard((B, T, C))
+    g2.attention_forward(out, None, None, dq, B, T, C, NH)
+    torch.cuda.synchronize()
+    check_guard(full, opad)
+    assert torch.isfinite(out).all()
+    assert_close(out, oracle.attention_forward(qkv, NH), "attention ragged")
 
 
 @pytest.mark.parametrize("B,T,NH,hs", [(2, 40, 4, 32), (1, 70, 2, 16), (1, 9, 3, 128), (2, 65, 2, 20)])
