@@ -684,6 +684,26 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   // from any cache: its tiles are stored with streaming stores, so that they do not push
   // the operands that other tiles are about to re-read out of L2.
   const bool stream_out = (size_t)M * N * sizeof(float) > ((size_t)256 << 20);
+  if (full && stream_out) {
+    // Row by row: the wave's TN segments of 128 bytes of one row go out back to back, as one run
+    // of TN * 128 bytes.  Rows of such a product (N = 50257) start at any multiple of 4 bytes, so
+    // every segment straddles memory lines; segments of one row that reach the L2 together are
+    // merged there, and only the two ends of the run are left as partial lines.
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      float* const o = out + (size_t)(m0 + wm * WM + i * 32 + 4 * h) * N + n0 + wn * WN + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          float r = acc[i][j][v];
+          if (GELU) r = gelu_tanh(r);
+          __builtin_nontemporal_store(r, o + (size_t)(8 * (v >> 2) + (v & 3)) * N + j * 32);
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -691,14 +711,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
       const int col = n0 + wn * WN + j * 32 + (lane & 31);
       const int rbase = m0 + wm * WM + i * 32 + 4 * h;
       float* o = out + (size_t)rbase * N + col;
-      if (full && stream_out) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          float r = acc[i][j][v];
-          if (GELU) r = gelu_tanh(r);
-          __builtin_nontemporal_store(r, o + (size_t)(8 * (v >> 2) + (v & 3)) * N);
-        }
-      } else if (full) {
+      if (full) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           float r = acc[i][j][v];

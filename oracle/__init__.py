@@ -14,7 +14,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+# ORACLE_LIB: another build of the same source to check against (the sanitizer build of the Makefile)
+_LIB_PATH = os.environ.get("ORACLE_LIB") or os.path.join(_HERE, "liboracle.so")
 _lib = None
 
 _f32p = ctypes.POINTER(ctypes.c_float)

@@ -243,6 +243,66 @@ def test_gpt2_graph_replays_with_k_split_gemms():
         model.close()
 
 
+def test_gpt2_graph_capture_and_replay_after_every_gemm_form_has_been_used():
+    """The launchers raise a kernel's dynamic-LDS limit the first time a thread uses it and
+    remember the kernels they have done it for (a table that used to hold 64 of them and now
+    grows).  Every tiled GEMM form the library has is touched first -- each tile shape, with and
+    without GELU, with and without a K split, the probed and the argmax forms -- then a forward
+    pass is captured and replayed: the capture must not contain (or trip over) an attribute call,
+    and the replays must give the eager result."""
+    import oracle as _oracle
+    ws = g2.matmul_forward_splitk_workspace()
+    M, C, OC = 320, 128, 448
+    r = np.random.default_rng(77)
+    x = torch.from_numpy(r.standard_normal((M, C), dtype=np.float32)).cuda()
+    w = torch.from_numpy((r.standard_normal((OC, C)) * 0.05).astype(np.float32)).cuda()
+    b = torch.from_numpy((r.standard_normal(OC) * 0.05).astype(np.float32)).cuda()
+    want = _oracle.matmul_forward(x.cpu().numpy(), w.cpu().numpy(), b.cpu().numpy())
+    out = torch.empty((M, OC), device="cuda")
+    forms = 0
+    for tile in ((256, 192), (256, 128), (128, 192), (128, 128), (128, 96), (64, 128), (64, 96), (64, 64), (32, 32)):
+        for splits in (1, 2):
+            for gelu in (False, True):
+                g2.matmul_forward_splitk(out, x, w, b, 1, M, C, OC, ws, is_gelu=gelu, plan=(*tile, splits))
+                forms += 1
+            torch.cuda.synchronize()
+        g2.matmul_forward_splitk(out, x, w, b, 1, M, C, OC, ws, plan=(*tile, 1))
+        torch.cuda.synchronize()
+        assert np.abs(out.cpu().numpy() - want).max() <= 1e-4, tile
+    # many 64x64 tiles take the two-buffer kernel instead of the ring (two more forms), many
+    # 128x192 tiles the four-wave form, K % 32 != 0 the register-staged kernel
+    big = torch.empty((2048, 1024), device="cuda")
+    xb = torch.randn(2048, 128, device="cuda")
+    wb = torch.randn(1024, 128, device="cuda") * 0.05
+    for gelu in (False, True):
+        g2.matmul_forward_splitk(big, xb, wb, None, 1, 2048, 128, 1024, ws, is_gelu=gelu, plan=(64, 64, 1))
+        g2.matmul_forward_gelu(out, x[:, :100].contiguous(), w[:, :100].contiguous(), b, 1, M, 100, OC, gelu)
+        forms += 2
+    g2.matmul_forward_probe(out, x, w, b, 1, M, C, OC)
+    ids_out = torch.empty(M, dtype=torch.int32, device="cuda")
+    g2.matmul_forward_argmax(ids_out, x, w, b, 1, M, C, OC)
+    forms += 2
+    torch.cuda.synchronize()
+    print(f"  {forms} GEMM forms used before the capture", flush=True)
+    assert int(ws[:g2.SPLITK_COUNTER_BYTES].max()) == 0
+
+    cfg = dict(max_seq_len=64, vocab_size=211, num_layers=2, num_heads=4, channels=256)
+    model = g2.GPT2(**cfg)
+    try:
+        model.load_params(syn.make_params(57, perturb_affine=True, **cfg))
+        ids = torch.from_numpy(syn.make_tokens(58, 2, 48, 211)).cuda()
+        model.forward(ids)
+        eager = model.logits().clone()
+        for rep in range(3):
+            model.forward_graph(ids)
+            torch.cuda.synchronize()
+            assert torch.equal(model.logits(), eager), f"replay {rep}"
+            g2.matmul_forward_splitk(out, x, w, b, 1, M, C, OC, ws, plan=(64, 96, 2))   # eager work between
+            torch.cuda.synchronize()
+    finally:
+        model.close()
+
+
 def test_launchers_follow_the_selected_stream():
     cfg = dict(max_seq_len=64, vocab_size=211, num_layers=2, num_heads=2, channels=128)
     model = g2.GPT2(**cfg)
