@@ -619,7 +619,9 @@ def main():
         for r in result["standalone"]:
             log("  standalone", json.dumps(r))
         # the path's next caller: incremental decoding against a key/value cache
-        result["decode"] = decode_bench(model, cfg, B, 128, 64)
+        # (a row per batch size: up to 16 sequences one persistent kernel per step, beyond that
+        # one launch per operation either way)
+        result["decode"] = [decode_bench(model, cfg, b, 128, 64) for b in (1, 8, 16, 32, 64)]
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(model, cfg, B, T)
         log("  cpu_baseline", json.dumps(result["cpu_baseline"]))

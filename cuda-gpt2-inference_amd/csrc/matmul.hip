@@ -1374,7 +1374,8 @@ static const TileCand kTileCands[] = {
     {128, 96, 1.017, 1.84, 1.93, 2.73, 0.54, 0.066},   {64, 128, 1.042, 2.08, 1.01, 2.30, 0.41, 0.0},
     {64, 64, 1.159, 0.40, 1.88, 1.65, 0.22, 0.115},    {32, 32, 1.398, 0.0, 3.54, 0.81, 0.20, 0.492},
     {64, 96, 1.094, 0.98, 3.06, 1.53, 0.44, 0.161},    {256, 192, 0.970, 7.5, 4.9, 1e9, 0.0, 0.0},
-    {256, 128, 1.000, 2.8, 4.0, 1e9, 0.0, 0.0}};
+    {256, 128, 1.000, 2.8, 4.0, 1e9, 0.0, 0.0},   {128, 160, 1.000, 4.6, 0.5, 4.0, 0.8, 0.05}};
+constexpr int kTile128x160 = 9;  // only for products whose width is a multiple of 160 (see choose_tile)
 // (256x192 -- eight waves of 64x96 -- moves 30 % fewer bytes into LDS per MFMA than 128x192 and
 // wins 1.5-2.5 points where its tiles come out in whole rounds: fc at M = 4096 / 8192, the
 // 350M qkv at 4096 / 8192.  256x128 -- eight waves of 64x64 -- does the same against 128x128 for
@@ -1410,6 +1411,10 @@ static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only, size_
   int best = 0, split_best = -1, split_parts = 1;
   double best_cost = 0, split_cost = 0;
   for (int i = 0; i < (two_largest_only ? 2 : kTileCandCount); i++) {
+    // 128x160 exists for the widths that no other shape divides into whole rounds (1280 = 8 x 160:
+    // GPT-2 large's projections at B*T = 4096 are 256 such tiles, against 224 ragged ones of
+    // 128x192 or 320 of 128x128); the GPT-2 124M / 350M widths are no multiples of 160
+    if (i == kTile128x160 && OC % 160 != 0) continue;
     const long long t = tiles_of(i, M, OC);
     TileCand c = kTileCands[i];
     const double work_us = 2.0 * c.bm * c.bn * (double)C / kCuFlopsPerUs;
@@ -1455,6 +1460,9 @@ static int launch_choice(int best, long long best_tiles, float* out, const float
                          const float* bias, int M, int C, int OC, bool gelu, unsigned long long* probe,
                          SplitK sk) {
   switch (best) {
+    case kTile128x160:
+      // four waves of 32x160, two workgroups per compute unit
+      return launch_dma<128, 160, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
     case 8:
       // eight waves of 64x64, one workgroup per compute unit
       return launch_dma<256, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);

@@ -82,7 +82,8 @@ void matmul_forward(float* out, const float* inp, const float* weight, const flo
                     int T, int C, int OC);
 
 /* Which workgroup tile (rows x columns of the product) matmul_forward gives a problem:
- * 256x192, 256x128, 128x192, 128x128, 128x96, 64x128, 64x96, 64x64 or 32x32, chosen by a fitted
+ * 256x192, 256x128, 128x192, 128x160 (only where OC is a multiple of 160), 128x128, 128x96,
+ * 64x128, 64x96, 64x64 or 32x32, chosen by a fitted
  * cost model so that the tiles come out in close to whole rounds over the 256 compute units
  * (the reference launches one fixed 128x128 tile shape and asserts divisibility,
  * kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:266-274).  Both are 0 for problems that

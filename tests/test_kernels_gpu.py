@@ -245,6 +245,8 @@ def test_matmul_bias(M, C, OC):
     (2048, 768, 3072, (128, 192)), (500, 768, 768, (32, 32)),
     (4096, 768, 3072, (256, 192)), (4090, 1024, 3070, (256, 192)),
     (8190, 768, 3070, (256, 192)), (2040, 1024, 4090, (256, 128)),
+    # widths that are multiples of 160 (GPT-2 large: 1280 channels): 128x160, with ragged rows
+    (4096, 1280, 1280, (128, 160)), (4090, 1280, 3840, (128, 160)), (2045, 1600, 4800, (128, 160)),
 ])
 def test_matmul_every_tile_shape_with_edges(M, C, OC, tile):
     say(f"matmul M={M} C={C} OC={OC} tile={tile}")
@@ -266,6 +268,7 @@ SPLITK_CASES = [
     (2048, 768, 2304, (128, 192), 2),
     (2048, 768, 768, (64, 96), 1), (2045, 768, 771, (64, 96), 2), (700, 3072, 2300, (64, 96), 5),
     (1000, 768, 1000, (256, 192), 1), (500, 1024, 380, (256, 192), 3), (700, 768, 250, (256, 128), 2),
+    (1000, 768, 1270, (128, 160), 1), (500, 1280, 1280, (128, 160), 3), (129, 96, 161, (128, 160), 2),
 ]
 
 
