@@ -473,11 +473,15 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode_kernel(
 // in flight; position t = 4 * (wave + 16 * i) + lane / 16.
 constexpr int DEC_UNROLL = 8;
 
-__global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
+// WAVES: waves per workgroup.  Sixteen keep the most rows in flight for one (sequence, head); with
+// more of those than the device holds such workgroups at once (two per compute unit), eight-wave
+// workgroups are all resident together instead of queueing for a second round.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES* kWave) void attention_decode64_kernel(
     float* __restrict__ out, const float* __restrict__ qkv, float* __restrict__ kc,
     float* __restrict__ vc, int pos, int maxT, int NH, float scale) {
   extern __shared__ float dec_lds[];  // scores [pos+1 rounded up to 64] | partial outputs [16][64]
-  __shared__ float red[2 * DEC_WAVES];
+  __shared__ float red[2 * WAVES];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -499,16 +503,16 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
   __syncthreads();  // the appended row is visible to the whole workgroup
 
   float mx = -INFINITY;
-  for (int g0 = wave; 4 * g0 <= pos; g0 += DEC_UNROLL * DEC_WAVES) {
+  for (int g0 = wave; 4 * g0 <= pos; g0 += DEC_UNROLL * WAVES) {
     f32x4 kf[DEC_UNROLL];
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
-      const int t = min(4 * (g0 + u * DEC_WAVES) + p4, pos);
+      const int t = min(4 * (g0 + u * WAVES) + p4, pos);
       kf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb + (size_t)t * 64));
     }
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
-      const int t = 4 * (g0 + u * DEC_WAVES) + p4;
+      const int t = 4 * (g0 + u * WAVES) + p4;
       const f32x4 pr = q4 * kf[u];
       const float s = row16_sum((pr[0] + pr[1]) + (pr[2] + pr[3])) * scale;
       if (t <= pos) {
@@ -523,28 +527,28 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
   __syncthreads();
   float m = red[0];
 #pragma unroll
-  for (int w = 1; w < DEC_WAVES; w++) m = fmaxf(m, red[w]);  // finite: position 0 always exists
+  for (int w = 1; w < WAVES; w++) m = fmaxf(m, red[w]);  // finite: position 0 always exists
 
   float sum = 0.f;
-  for (int t = tid; t <= pos; t += DEC_WAVES * kWave) {
+  for (int t = tid; t <= pos; t += WAVES * kWave) {
     const float e = expf(sc[t] - m);
     sc[t] = e;
     sum += e;
   }
   sum = wave_sum(sum);
-  if (lane == 0) red[DEC_WAVES + wave] = sum;
+  if (lane == 0) red[WAVES + wave] = sum;
   __syncthreads();
   float l = 0.f;
 #pragma unroll
-  for (int w = 0; w < DEC_WAVES; w++) l += red[DEC_WAVES + w];
+  for (int w = 0; w < WAVES; w++) l += red[WAVES + w];
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int g0 = wave; 4 * g0 <= pos; g0 += DEC_UNROLL * DEC_WAVES) {
+  for (int g0 = wave; 4 * g0 <= pos; g0 += DEC_UNROLL * WAVES) {
     f32x4 vf[DEC_UNROLL];
     float pw[DEC_UNROLL];
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
-      const int t = 4 * (g0 + u * DEC_WAVES) + p4;
+      const int t = 4 * (g0 + u * WAVES) + p4;
       pw[u] = (t <= pos) ? sc[t] : 0.f;
       vf[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb + (size_t)min(t, pos) * 64));
     }
@@ -561,7 +565,7 @@ __global__ __launch_bounds__(DEC_WAVES* kWave) void attention_decode64_kernel(
   if (tid < 64) {
     float o = 0.f;
 #pragma unroll
-    for (int w = 0; w < DEC_WAVES; w++) o += part[w * 64 + tid];
+    for (int w = 0; w < WAVES; w++) o += part[w * 64 + tid];
     out[(size_t)b * C + head * 64 + tid] = o / l;
   }
 }
@@ -595,8 +599,12 @@ int attention_decode_launch(float* out, const float* qkv, float* kc, float* vc, 
   if (lds > 60 * 1024)
     return fail(GPT2HIP_EINVAL, "attention_decode: position %d needs %zu bytes of LDS", pos, lds);
   if (hs == 64 && aligned16(qkv) && aligned16(kc) && aligned16(vc))
-    hipLaunchKernelGGL(attention_decode64_kernel, dim3((unsigned)(B * NH)), dim3(DEC_WAVES * kWave), lds,
-                       stream(), out, qkv, kc, vc, pos, maxT, NH, 1.0f / sqrtf(64.f));
+    if (B * NH > 512)
+      hipLaunchKernelGGL(attention_decode64_kernel<8>, dim3((unsigned)(B * NH)), dim3(8 * kWave), lds, stream(), out,
+                         qkv, kc, vc, pos, maxT, NH, 1.0f / sqrtf(64.f));
+    else
+      hipLaunchKernelGGL(attention_decode64_kernel<DEC_WAVES>, dim3((unsigned)(B * NH)), dim3(DEC_WAVES * kWave), lds,
+                         stream(), out, qkv, kc, vc, pos, maxT, NH, 1.0f / sqrtf(64.f));
   else
     hipLaunchKernelGGL(attention_decode_kernel, dim3((unsigned)(B * NH)), dim3(DEC_WAVES * kWave), lds,
                        stream(), out, qkv, kc, vc, pos, maxT, NH, hs, 1.0f / sqrtf((float)hs));
