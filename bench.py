@@ -400,11 +400,18 @@ def decode_bench(model, cfg, B, T0, steps):
         model.prefill(ids)
         torch.cuda.synchronize()
         out["prefill_ms"] = (time.perf_counter() - t0) * 1e3
-        t0 = time.perf_counter()
-        for i in range(steps):
-            model.decode(nxt[4 + i])
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) / steps * 1e3
+        # three runs of `steps` steps from the same prompt, the median one reported: the first run
+        # after the cache has been (re)allocated for another batch size is now and then much slower
+        runs = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for i in range(steps):
+                model.decode(nxt[4 + i])
+            torch.cuda.synchronize()
+            runs.append((time.perf_counter() - t0) / steps * 1e3)
+            model.prefill(ids)
+            torch.cuda.synchronize()
+        ms = sorted(runs)[1]
         gbs = (weight_bytes + cache_bytes) / ms / 1e6
         out[name] = {"ms_per_step": ms, "tokens_per_s": B / ms * 1e3, "GB/s": gbs,
                      "frac_hbm": gbs / PEAK_HBM_GBS,

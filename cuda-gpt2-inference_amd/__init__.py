@@ -427,8 +427,8 @@ class GPT2:
         return cls(_handle=h, **cfg)
 
     def close(self):
-        if getattr(self, "_h", None):
-            lib().gpt2_destroy(self._h)
+        if getattr(self, "_h", None) and _lib is not None:  # at interpreter exit the module may be gone
+            _lib.gpt2_destroy(self._h)
             self._h = None
 
     __del__ = close
