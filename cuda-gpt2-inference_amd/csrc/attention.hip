@@ -76,7 +76,7 @@ __device__ __forceinline__ float pair_sum(float x) {
 template <int P, bool RAGGED>
 __global__ __launch_bounds__(ATT_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ qkv, int T, int NH,
-                            int nqb, float scale_log2e) {
+                            int nqb, float scale_log2e, int snake) {
   constexpr int QG = ATT_WAVES / P;  // query groups per workgroup
   constexpr int BQ = 32 * QG;        // queries per workgroup
   __shared__ __attribute__((aligned(16))) char lds_all[ATT_WAVES * WAVE_LDS_BYTES];
@@ -87,8 +87,17 @@ void attention_flash_kernel(float* __restrict__ out, const float* __restrict__ q
   const int h32 = lane >> 5;
   const int l32 = lane & 31;
 
-  // heaviest query blocks (most keys) are launched first
-  const int bid = blockIdx.x;
+  // Heaviest query blocks (most keys) first.  When all workgroups are resident at once (three per
+  // compute unit) nothing is handed out dynamically: the dispatcher deals workgroup ids breadth
+  // first, ids i, i + CUs, i + 2 CUs to the same compute unit, which in descending order of weight
+  // gives one unit the heaviest of every third and another the lightest (17 against 10 sub-tiles
+  // at B=8, T=256, NH=12).  `snake` (the number of compute units, or 0) deals every second row of
+  // ids in reverse instead, as one deals out cards by strength.
+  int bid = blockIdx.x;
+  if (snake > 0) {
+    const int row = bid / snake, first = row * snake;
+    if (row & 1) bid = first + (min(snake, (int)gridDim.x - first) - 1 - (bid - first));
+  }
   const int per_block = gridDim.x / nqb;  // = B*NH
   const int qblock = nqb - 1 - bid / per_block;
   const int bh = bid % per_block;
@@ -655,8 +664,14 @@ int attention_forward_status(float* out, float* qkvr, float* att, const float* i
     const bool ragged = T % 32 != 0;
     auto kfn = P == 2 ? (ragged ? attention_flash_kernel<2, true> : attention_flash_kernel<2, false>)
                       : (ragged ? attention_flash_kernel<4, true> : attention_flash_kernel<4, false>);
+    // all workgroups resident at once (three per compute unit): see the kernel's `snake`
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      cus = 0;
+    const int snake = (cus > 0 && blocks <= 3LL * cus) ? cus : 0;
     hipLaunchKernelGGL(kfn, dim3((unsigned)blocks), dim3(ATT_THREADS), 0, stream(), out, inp, T, NH, nqb,
-                       scale_log2e);
+                       scale_log2e, snake);
   } else {
     if (hs > 256) return fail(GPT2HIP_EINVAL, "attention_forward: head size %d > 256", hs);
     const long long waves = (long long)B * NH * T;
