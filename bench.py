@@ -580,6 +580,11 @@ def main():
                         "frac_hbm_net_of_marker": nbytes[k] / net / 1e6 / PEAK_HBM_GBS,
                         "note": "inside the forward pass, operands may be served by the 256 MiB "
                                 "Infinity Cache"})
+        if k == "encoder":
+            row["note"] = ("the pass's first launch: its interval also holds the opening event's own trip and "
+                           "the host's launch latency (the device finishes the untimed launches in front of it "
+                           "before the host has queued the next one); the kernel by itself is the "
+                           "encoder_forward row of standalone[]")
         kernels.append(row)
         log(f"  {k:26s} {prof[k]:8.3f} ms/fwd  " + (f"{row.get('TFLOP/s', 0):7.1f} TFLOP/s"
             if k in flops else f"{row.get('GB/s', 0):7.0f} GB/s"))

@@ -242,14 +242,21 @@ static const char* const kProfNames[GPT2_PROF_COUNT] = {
     "matmul_forward lm-head"};
 
 struct Profile {
-  std::vector<hipEvent_t> events;
+  std::vector<hipEvent_t> events;  // the first `used` of them have been recorded
   std::vector<int> category;
+  size_t used = 0;
+  int reserve(size_t n) {
+    while (events.size() < n) {
+      hipEvent_t e;
+      G2_HIP(hipEventCreate(&e));
+      events.push_back(e);
+    }
+    return GPT2HIP_OK;
+  }
   int mark(int cat) {  // cat < 0: the opening event
-    hipEvent_t e;
-    G2_HIP(hipEventCreate(&e));
-    events.push_back(e);
+    if (int rc = reserve(used + 1)) return rc;
     if (cat >= 0) category.push_back(cat);
-    G2_HIP(hipEventRecord(e, stream()));
+    G2_HIP(hipEventRecord(events[used++], stream()));
     return GPT2HIP_OK;
   }
   ~Profile() {
@@ -846,14 +853,14 @@ int gpt2_forward_profiled_status(GPT2* model, const int* inputs_device, int B, i
   // then sits between back-to-back launches like every other event of the pass, instead of
   // behind the copy of the ids and the device's wake-up from idle, and the device is still busy
   // with them while the host queues that event and the first timed launch.
+  Profile prof;
   for (int i = 0; i < 4; i++)
     if (int rc = encoder_launch(model->res_a, model->ids, model->params + model->param_off[P_WTE],
                                 model->params + model->param_off[P_WPE], B, T, model->cfg.channels,
                                 model->cfg.vocab_size))
       return rc;
-  Profile prof;
   if (int rc = forward_resident(model, B, T, &prof)) return rc;
-  G2_HIP(hipEventSynchronize(prof.events.back()));
+  G2_HIP(hipEventSynchronize(prof.events[prof.used - 1]));
   for (int i = 0; i < GPT2_PROF_COUNT; i++) ms_per_category[i] = 0.f;
   for (size_t i = 0; i < prof.category.size(); i++) {
     float ms = 0.f;
@@ -881,16 +888,16 @@ float gpt2hip_profile_marker_overhead_us(int launches) {
     if (prof.mark(-1)) break;
     bool ok = true;
     for (int i = 0; i < launches && ok; i++) ok = !residual_forward_status(buf, buf, buf, 256) && !prof.mark(0);
-    if (!ok || hipEventSynchronize(prof.events.back()) != hipSuccess) break;
+    if (!ok || hipEventSynchronize(prof.events[prof.used - 1]) != hipSuccess) break;
     float marked = 0.f;
-    if (hipEventElapsedTime(&marked, prof.events.front(), prof.events.back()) != hipSuccess) break;
+    if (hipEventElapsedTime(&marked, prof.events.front(), prof.events[prof.used - 1]) != hipSuccess) break;
     // (b) the same launches back to back between two events
     Profile bare;
     if (bare.mark(-1)) break;
     for (int i = 0; i < launches && ok; i++) ok = !residual_forward_status(buf, buf, buf, 256);
-    if (!ok || bare.mark(0) || hipEventSynchronize(bare.events.back()) != hipSuccess) break;
+    if (!ok || bare.mark(0) || hipEventSynchronize(bare.events[bare.used - 1]) != hipSuccess) break;
     float plain = 0.f;
-    if (hipEventElapsedTime(&plain, bare.events.front(), bare.events.back()) != hipSuccess) break;
+    if (hipEventElapsedTime(&plain, bare.events.front(), bare.events[bare.used - 1]) != hipSuccess) break;
     result = (marked - plain) * 1000.f / (float)launches;
     if (result < 0.f) result = 0.f;
   } while (false);
