@@ -465,7 +465,10 @@ def test_matmul_probe_rejects_small_buffer_and_odd_k():
 # ------------------------------------------------------------------ attention
 @pytest.mark.parametrize("B,T,NH", [(8, 1024, 12), (8, 256, 12), (8, 1024, 16), (8, 256, 16),
                                     (2, 1024, 16), (4, 256, 16), (4, 64, 12), (1, 1, 2), (2, 33, 3),
-                                    (1, 130, 2), (1, 200, 1), (3, 512, 5), (1, 448, 12)])
+                                    (1, 130, 2), (1, 200, 1), (3, 512, 5), (1, 448, 12),
+                                    # all workgroups resident at once, dealt to the compute units in
+                                    # alternating direction: three full rows of 256, a partial second row
+                                    (2, 1024, 12), (1, 1024, 12), (5, 160, 13)])
 def test_attention_hs64(B, T, NH):
     say(f"attention B={B} T={T} NH={NH} HS=64")
     C = NH * 64
