@@ -84,12 +84,16 @@ def forward_flops(cfg, B, T):
     return per_forward
 
 
-def forward_bytes(cfg, B, T):
+def forward_bytes(cfg, B, T, sums_in_matmul):
+    """Algorithmic bytes per forward of the memory-bound launches.  Where the driver forms the
+    residual sums in the projections' epilogues, the normalisation that follows reads the sum
+    and writes its normalisation (8 bytes per entry) instead of reading two rows and writing
+    two (16)."""
     C, L = cfg["channels"], cfg["num_layers"]
     M = B * T
     return {"encoder": 4 * M + 8 * M * C + 4 * T * C,
             "layernorm": 8 * M * C + 8 * C,
-            "fused_residual_layernorm": 2 * L * (16 * M * C + 8 * C)}
+            "fused_residual_layernorm": 2 * L * ((8 if sums_in_matmul else 16) * M * C + 8 * C)}
 
 
 LAUNCHES = {"encoder": 1, "layernorm": 1, "matmul_lmhead": 1}
@@ -228,6 +232,24 @@ def standalone(g2):
                     "note": f"tile {plan[0]}x{plan[1]}, K split {plan[2]} ways; matmul_forward "
                             f"(no workspace): {ms_plain:.4f} ms"})
         del x, w, o
+    # the two projections with the block's residual add in their epilogue, as the driver runs
+    # them at this size (out = resid + product), beside the plain product of the same shape
+    for (C, OC) in ((768, 768), (3072, 768)):
+        x = torch.randn(M, C, device=dev)
+        w = torch.randn(OC, C, device=dev) * 0.02
+        bb = torch.randn(OC, device=dev) * 0.02
+        r = torch.randn(M, OC, device=dev)
+        o = torch.empty(M, OC, device=dev)
+        a = (P(o), P(x), P(w), P(bb), P(r), 8, 1024, C, OC, P(ws), ws.numel())
+        ms = time_launch(g2, lambda i: L.matmul_forward_residual_status(*a), iters=40)
+        ms_plain = time_launch(g2, lambda i: L.matmul_forward(*a[:4], *a[5:9]), iters=40)
+        tf = 2.0 * M * C * OC / ms / 1e9
+        out.append({"kernel": "matmul_forward_residual", "shape": f"M={M},C={C},OC={OC}", "ms": ms,
+                    "TFLOP/s": tf, "frac_fp32_mfma": tf / PEAK_FP32_MFMA_TFLOPS,
+                    "note": f"matmul_forward of the same shape in the same loop: {ms_plain:.4f} ms; the "
+                            "add saves the normalisation kernel behind it half its traffic "
+                            "(layernorm_forward against fused_residual_layernorm below)"})
+        del x, w, o, r
     # causal attention
     for (B, T, NH) in ((8, 1024, 12), (8, 256, 12), (8, 1024, 16), (8, 256, 16)):
         C = NH * 64
@@ -558,7 +580,8 @@ def main():
             prof[k] += v
     prof = {k: v / args.steps for k, v in prof.items()}   # ms per forward per category
     flops = forward_flops(cfg, B, T)
-    nbytes = forward_bytes(cfg, B, T)
+    sums_in_matmul = g2.forward_sums_in_matmul(cfg, B, T)
+    nbytes = forward_bytes(cfg, B, T, sums_in_matmul)
     L = cfg["num_layers"]
     marker_ms = marker_overhead_ms(g2)
     log(f"  event marker between two launches: +{marker_ms * 1e3:.2f} us per interval")
@@ -580,6 +603,12 @@ def main():
                         "frac_hbm_net_of_marker": nbytes[k] / net / 1e6 / PEAK_HBM_GBS,
                         "note": "inside the forward pass, operands may be served by the 256 MiB "
                                 "Infinity Cache"})
+        if sums_in_matmul and k == "fused_residual_layernorm":
+            row["note"] = ("at this size the driver adds the residual stream in the epilogues of the two "
+                           "projections (matmul_forward_residual_status) and these launches are "
+                           "layernorm_forward on the sum: 8 bytes per entry instead of 16; " + row["note"])
+        if sums_in_matmul and k in ("matmul_attproj", "matmul_fcproj"):
+            row["note"] = "out = residual + product: the block's residual add is in this launch's epilogue"
         if k == "encoder":
             row["note"] = ("the pass's first launch: its interval also holds the opening event's own trip and "
                            "the host's launch latency (the device finishes the untimed launches in front of it "

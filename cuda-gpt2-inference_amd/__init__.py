@@ -43,6 +43,7 @@ EXPORTS = (
     "matmul_forward_tile_shape",
     "matmul_forward_splitk_workspace", "matmul_forward_splitk_status",
     "matmul_forward_splitk_plan", "matmul_forward_splitk_forced_status",
+    "matmul_forward_residual_status",
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
     "matmul_forward_argmax_workspace", "matmul_forward_argmax_status",
@@ -53,7 +54,7 @@ EXPORTS = (
     "gpt2_forward_device_status", "gpt2_forward_graph_status",
     "gpt2_prefill_status", "gpt2_decode_status", "gpt2_decode_sync_status", "gpt2_decode_options", "gpt2_decode_probe_status", "gpt2_decode_probe_size",
     "gpt2_step_logits", "gpt2_cache_length",
-    "gpt2_forward_argmax_status",
+    "gpt2_forward_argmax_status", "gpt2_forward_sums_in_matmul",
     "gpt2_forward_profiled_status", "gpt2hip_profile_marker_overhead_us", "gpt2_logits", "gpt2_lnf", "gpt2_argmax_status",
     "gpt2hip_timer_create", "gpt2hip_timer_destroy", "gpt2hip_timer_start",
     "gpt2hip_timer_stop_ms",
@@ -144,6 +145,8 @@ def lib() -> ctypes.CDLL:
         L.matmul_forward_splitk_status.restype = ci
         L.matmul_forward_splitk_forced_status.argtypes = [vp] * 4 + [ci] * 5 + [vp, cz] + [ci] * 3
         L.matmul_forward_splitk_forced_status.restype = ci
+        L.matmul_forward_residual_status.argtypes = [vp] * 5 + [ci] * 4 + [vp, cz]
+        L.matmul_forward_residual_status.restype = ci
         L.matmul_forward_splitk_plan.argtypes = [ci] * 4 + [cz] + [ctypes.POINTER(ci)] * 3
         L.matmul_forward_splitk_plan.restype = ci
         L.gpt2_create.argtypes, L.gpt2_create.restype = [ctypes.POINTER(GPT2Config)], vp
@@ -173,6 +176,8 @@ def lib() -> ctypes.CDLL:
         L.gpt2hip_set_stream.argtypes, L.gpt2hip_set_stream.restype = [vp], None
         L.gpt2hip_get_stream.argtypes, L.gpt2hip_get_stream.restype = [], vp
         L.gpt2hip_set_workspace.argtypes, L.gpt2hip_set_workspace.restype = [vp, cz], ci
+        L.gpt2_forward_sums_in_matmul.argtypes = [ctypes.POINTER(GPT2Config), ci, ci]
+        L.gpt2_forward_sums_in_matmul.restype = ci
         L.gpt2_forward_argmax_status.argtypes = [vp, vp, ci, ci, vp]
         L.gpt2_forward_argmax_status.restype = ci
         L.matmul_forward_argmax_workspace.argtypes = [ci, ci, ci]
@@ -313,6 +318,22 @@ def matmul_forward_splitk(out, inp, weight, bias, B, T, C, OC, workspace, is_gel
                                                          _f32(bias), B, T, C, OC, int(bool(is_gelu)),
                                                          ws, nbytes, *map(int, plan)),
                "matmul_forward_splitk_forced")
+
+
+def matmul_forward_residual(out, inp, weight, bias, resid, B, T, C, OC, workspace=None):
+    """out = resid + (inp . weight^T + bias), the residual add in the product's epilogue.
+    workspace: as for matmul_forward_splitk (None: K is not split between workgroups)."""
+    ws, nbytes = (None, 0) if workspace is None else (workspace.data_ptr(), workspace.numel())
+    _check(lib().matmul_forward_residual_status(_f32(out), _f32(inp), _f32(weight), _f32(bias),
+                                                _f32(resid), B, T, C, OC, ws, nbytes),
+           "matmul_forward_residual")
+
+
+def forward_sums_in_matmul(config, B, T):
+    """Whether gpt2_forward at this size adds the residual stream in the projections' epilogues
+    (config: a dict with the GPT2Config fields, e.g. GPT2_124M).  No GPU needed."""
+    cfg = GPT2Config(**config)
+    return bool(lib().gpt2_forward_sums_in_matmul(ctypes.byref(cfg), B, T))
 
 
 def matmul_forward_splitk_plan(B, T, C, OC, workspace_bytes):

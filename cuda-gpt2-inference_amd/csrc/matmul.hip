@@ -119,6 +119,82 @@ __device__ __forceinline__ void argmax_fold(float* bv, int* bx, int lane, int& f
   }
 }
 
+// The epilogue the tiled kernels share: a wave's TM x TN accumulator tiles go to out (through
+// GELU if asked), plus resid's entries of the same positions where resid is given (the residual
+// add of a transformer block, which then needs no pass of its own over memory: out = resid +
+// act(product); out and resid must not overlap).  row0 / col0: this lane's first row and its
+// column in the wave's first tile.  All of a wave's loads of resid are issued before its first
+// store.
+// (a full tile's entries of resid, in the accumulators' layout)
+template <int TM, int TN>
+__device__ __forceinline__ void load_resid_tile(f32x16 (&rs)[TM][TN], const float* __restrict__ resid,
+                                                int row0, int col0, int N) {
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const float* const rp = resid + (size_t)(row0 + i * 32) * N + col0 + j * 32;
+#pragma unroll
+      for (int v = 0; v < 16; v++) rs[i][j][v] = rp[(size_t)(8 * (v >> 2) + (v & 3)) * N];
+    }
+}
+// (a full tile: out = act(acc) + rs)
+template <int TM, int TN, bool GELU>
+__device__ __forceinline__ void store_tile_sum(const f32x16 (&acc)[TM][TN], const f32x16 (&rs)[TM][TN],
+                                               float* __restrict__ out, int row0, int col0, int N) {
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      float* const o = out + (size_t)(row0 + i * 32) * N + col0 + j * 32;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        float r = acc[i][j][v];
+        if (GELU) r = gelu_tanh(r);
+        o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r + rs[i][j][v];
+      }
+    }
+}
+template <int TM, int TN, bool GELU>
+__device__ __forceinline__ void store_tile(const f32x16 (&acc)[TM][TN], float* __restrict__ out,
+                                           const float* __restrict__ resid, int row0, int col0, int M,
+                                           int N, bool full) {
+  if (full && resid != nullptr) {
+    f32x16 rs[TM][TN];
+    load_resid_tile<TM, TN>(rs, resid, row0, col0, N);
+    store_tile_sum<TM, TN, GELU>(acc, rs, out, row0, col0, N);
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const int col = col0 + j * 32;
+      const int rbase = row0 + i * 32;
+      float* o = out + (size_t)rbase * N + col;
+      if (full) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          float r = acc[i][j][v];
+          if (GELU) r = gelu_tanh(r);
+          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
+        }
+      } else if (col < N) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int row = rbase + 8 * (v >> 2) + (v & 3);
+          if (row < M) {
+            float r = acc[i][j][v];
+            if (GELU) r = gelu_tanh(r);
+            if (resid != nullptr) r += resid[(size_t)row * N + col];
+            out[(size_t)row * N + col] = r;
+          }
+        }
+      }
+    }
+  }
+}
+
 // K split between workgroups.  The `splits` workgroups of a tile each multiply one
 // contiguous range of the K slabs and leave their partial tile (the raw accumulators, lane
 // by lane: [tile][part][wave][register quad][lane], 1 KB per store instruction) in a
@@ -191,7 +267,7 @@ __device__ __forceinline__ bool splitk_combine(f32x16 (&acc)[TM][TN], float* __r
 template <int BM, int BN, int WGM, int WGN, bool GELU, bool KTAIL>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn) {
+    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ntm, int ntn) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -376,33 +452,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
 
   // ---- epilogue -----------------------------------------------------------
   const bool full = (m0 + BM <= M) && (n0 + BN <= N);
-#pragma unroll
-  for (int i = 0; i < TM; i++) {
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const int col = n0 + wn * WN + j * 32 + (lane & 31);
-      const int rbase = m0 + wm * WM + i * 32 + 4 * h;
-      float* o = out + (size_t)rbase * N + col;
-      if (full) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          float r = acc[i][j][v];
-          if (GELU) r = gelu_tanh(r);
-          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
-        }
-      } else if (col < N) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const int row = rbase + 8 * (v >> 2) + (v & 3);
-          if (row < M) {
-            float r = acc[i][j][v];
-            if (GELU) r = gelu_tanh(r);
-            out[(size_t)row * N + col] = r;
-          }
-        }
-      }
-    }
-  }
+  store_tile<TM, TN, GELU>(acc, out, resid, m0 + wm * WM + 4 * h, n0 + wn * WN + (lane & 31), M, N, full);
 }
 
 // ---------------------------------------------------------------------------
@@ -435,11 +485,17 @@ typedef const __attribute__((address_space(1))) void glb_void_t;
 //
 // SPLIT: the grid is `splits` workgroups per tile (workgroup id = part * tiles + tile), each
 // taking slabs [part * nslab / splits, (part + 1) * nslab / splits); see splitk_combine.
+//
+// RESID: out = resid + product for a product whose tiles come in about one round (every compute
+// unit reaches its epilogue at the same moment, and B*T x OC floats of resid read there in one
+// burst cost 4-5 us that nothing hides).  Each wave fetches its part of the tile of resid into
+// registers during the slab loop instead, wave w two slabs earlier than wave w - 1, so that the
+// reads are spread over the loop's last slabs and are long there when the epilogue starts.
 template <int BM, int BN, int WGM, int WGN, bool GELU, bool PROBE = false, bool ARGMAX = false,
-          bool SPLIT = false>
+          bool SPLIT = false, bool RESID = false>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn,
+    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ntm, int ntn,
     unsigned long long* __restrict__ probe, int* __restrict__ arg_idx, float* __restrict__ part_ws,
     unsigned* __restrict__ part_cnt, int splits) {
   constexpr int NW = WGM * WGN;
@@ -614,12 +670,35 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     wall0 = wall_clock64();
     clk0 = clock64();
   }
+  // RESID: this wave's entries of resid (full tiles; an edge tile reads them in the epilogue)
+  const bool full = (m0 + BM <= M) && (n0 + BN <= N);
+  const int row0 = m0 + wm * WM + 4 * (lane >> 5), col0 = n0 + wn * WN + (lane & 31);
+  f32x16 rs[RESID ? TM : 1][RESID ? TN : 1];
+  const int resid_at = RESID && full ? max(0, nslab / 2 - 1 - wave) : -1;  // pair of slabs to fetch in front of
+  bool resid_loaded = false;
   int s = 0;
-  for (; s + 1 < nslab; s += 2) {
+  // (RESID: the last NW pairs of slabs run in a second copy of the loop, which is the one that
+  // carries the check for the wave's turn to fetch; the check in the loop itself cost every
+  // pair of slabs 70 ns)
+  const int s_check = RESID ? max(0, nslab / 2 - NW) * 2 : nslab;
+  for (; s + 1 < min(nslab, s_check); s += 2) {
     slab_body(s, std::integral_constant<int, 0>{});
     slab_body(s + 1, std::integral_constant<int, 1>{});
   }
+  if constexpr (RESID) {
+    for (; s + 1 < nslab; s += 2) {
+      if ((s >> 1) == resid_at) {
+        load_resid_tile<TM, TN>(rs, resid, row0, col0, N);
+        resid_loaded = true;
+      }
+      slab_body(s, std::integral_constant<int, 0>{});
+      slab_body(s + 1, std::integral_constant<int, 1>{});
+    }
+  }
   if (s < nslab) slab_body(s, std::integral_constant<int, 0>{});
+  if constexpr (RESID) {
+    if (full && !resid_loaded) load_resid_tile<TM, TN>(rs, resid, row0, col0, N);
+  }
   if (PROBE && tid == 0) {
     probe[4 * blockIdx.x + 0] = wall0;
     probe[4 * blockIdx.x + 1] = wall_clock64();
@@ -679,12 +758,17 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     }
     return;
   }
-  const bool full = (m0 + BM <= M) && (n0 + BN <= N);
+  if constexpr (RESID) {
+    if (full) {
+      store_tile_sum<TM, TN, GELU>(acc, rs, out, row0, col0, N);
+      return;
+    }
+  }
   // A product larger than the 256 MiB Infinity Cache (the logits) will not be read back
   // from any cache: its tiles are stored with streaming stores, so that they do not push
   // the operands that other tiles are about to re-read out of L2.
   const bool stream_out = (size_t)M * N * sizeof(float) > ((size_t)256 << 20);
-  if (full && stream_out) {
+  if (full && stream_out && resid == nullptr) {
     // Row by row: the wave's TN segments of 128 bytes of one row go out back to back, as one run
     // of TN * 128 bytes.  Rows of such a product (N = 50257) start at any multiple of 4 bytes, so
     // every segment straddles memory lines; segments of one row that reach the L2 together are
@@ -704,33 +788,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     }
     return;
   }
-#pragma unroll
-  for (int i = 0; i < TM; i++) {
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const int col = n0 + wn * WN + j * 32 + (lane & 31);
-      const int rbase = m0 + wm * WM + i * 32 + 4 * h;
-      float* o = out + (size_t)rbase * N + col;
-      if (full) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          float r = acc[i][j][v];
-          if (GELU) r = gelu_tanh(r);
-          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
-        }
-      } else if (col < N) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const int row = rbase + 8 * (v >> 2) + (v & 3);
-          if (row < M) {
-            float r = acc[i][j][v];
-            if (GELU) r = gelu_tanh(r);
-            out[(size_t)row * N + col] = r;
-          }
-        }
-      }
-    }
-  }
+  store_tile<TM, TN, GELU>(acc, out, resid, row0, col0, M, N, full);
 }
 
 // s_waitcnt immediate that waits until at most n vector-memory operations of this wave
@@ -756,7 +814,7 @@ template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool GELU, bool SP
           bool PIPE = false>
 __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, int M, int K, int N, int ntm, int ntn,
+    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ntm, int ntn,
     float* __restrict__ part_ws, unsigned* __restrict__ part_cnt, int splits) {
   constexpr int NMN = WGM * WGN;
   constexpr int NW = NMN * KS;
@@ -986,33 +1044,7 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
   }
 
   const bool full = (m0 + BM <= M) && (n0 + BN <= N);
-#pragma unroll
-  for (int i = 0; i < TM; i++) {
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const int col = n0 + wn * WN + j * 32 + (lane & 31);
-      const int rbase = m0 + wm * WM + i * 32 + 4 * h;
-      float* o = out + (size_t)rbase * N + col;
-      if (full) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          float r = acc[i][j][v];
-          if (GELU) r = gelu_tanh(r);
-          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
-        }
-      } else if (col < N) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const int row = rbase + 8 * (v >> 2) + (v & 3);
-          if (row < M) {
-            float r = acc[i][j][v];
-            if (GELU) r = gelu_tanh(r);
-            out[(size_t)row * N + col] = r;
-          }
-        }
-      }
-    }
-  }
+  store_tile<TM, TN, GELU>(acc, out, resid, m0 + wm * WM + 4 * h, n0 + wn * WN + (lane & 31), M, N, full);
 }
 
 // M <= 16 rows (one token per sequence: a decode step).  Such a product is bound by
@@ -1157,8 +1189,8 @@ int skinny_launch(float* out, const float* inp, const float* weight, const float
 // multiple of 4 or an operand is not 16-byte aligned.
 __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const float* inp,
                                                               const float* weight,
-                                                              const float* bias, int M, int K, int N,
-                                                              int gelu) {
+                                                              const float* bias, const float* resid,
+                                                              int M, int K, int N, int gelu) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (size_t)M * N) return;
   const int row = (int)(idx / N), col = (int)(idx % N);
@@ -1166,7 +1198,8 @@ __global__ __launch_bounds__(256) void matmul_generic_kernel(float* out, const f
   const float* w = weight + (size_t)col * K;
   float acc = bias ? bias[col] : 0.f;
   for (int k = 0; k < K; k++) acc += x[k] * w[k];
-  out[idx] = gelu ? gelu_tanh(acc) : acc;
+  acc = gelu ? gelu_tanh(acc) : acc;
+  out[idx] = resid ? acc + resid[idx] : acc;
 }
 
 // Reduces the (value, column) pairs that the ARGMAX form of matmul_dma_kernel leaves
@@ -1249,7 +1282,7 @@ static int allow_lds(const void* kfn, size_t lds_bytes) {
 // Register-staged kernel: any K % 4 == 0.
 template <int BM, int BN, int WGM, int WGN>
 static int launch_mfma(float* out, const float* inp, const float* weight, const float* bias, int M,
-                       int K, int N, bool gelu) {
+                       int K, int N, bool gelu, const float* resid = nullptr) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
@@ -1261,8 +1294,8 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
                    : (gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true, false>
                            : matmul_mfma_kernel<BM, BN, WGM, WGN, false, false>);
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
-                     K, N, ntm, ntn);
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, resid,
+                     M, K, N, ntm, ntn);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1278,7 +1311,8 @@ struct SplitK {
 // LDS-DMA kernel: K % 32 == 0.  The clock-probe form exists for PROBED tile shapes only.
 template <int BM, int BN, int WGM, int WGN, bool PROBED = false>
 static int launch_dma(float* out, const float* inp, const float* weight, const float* bias, int M,
-                      int K, int N, bool gelu, unsigned long long* probe = nullptr, SplitK sk = {}) {
+                      int K, int N, bool gelu, unsigned long long* probe = nullptr, SplitK sk = {},
+                      const float* resid = nullptr) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
@@ -1289,14 +1323,19 @@ static int launch_dma(float* out, const float* inp, const float* weight, const f
     if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: no probe form with K split");
     kfn = gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true, false, false, true>
                : matmul_dma_kernel<BM, BN, WGM, WGN, false, false, false, true>;
+  } else if (resid && !gelu && !probe && (BM / WGM / 32) * (BN / WGN / 32) <= 3) {
+    // (larger register tiles have no room for the tile of resid beside the accumulators: they read
+    // it in the epilogue)
+    if constexpr ((BM / WGM / 32) * (BN / WGN / 32) <= 3)
+      kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, false, false, false, true>;
   } else if constexpr (PROBED) {
     if (probe) kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, true>;
   } else if (probe) {
     return fail(GPT2HIP_EINVAL, "matmul_forward_probe: no probe form of the %dx%d tile", BM, BN);
   }
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
-                     K, N, ntm, ntn, probe, (int*)nullptr, sk.ws, sk.cnt, sk.splits);
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, resid,
+                     M, K, N, ntm, ntn, probe, (int*)nullptr, sk.ws, sk.cnt, sk.splits);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1313,8 +1352,8 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
   auto kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, false, true>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)(ntm * ntn)), dim3(NT), lds_bytes, stream(), pair_val, inp, weight,
-                     bias, M, K, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx, (float*)nullptr,
-                     (unsigned*)nullptr, 1);
+                     bias, (const float*)nullptr, M, K, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx,
+                     (float*)nullptr, (unsigned*)nullptr, 1);
   G2_LAUNCH_CHECK("matmul_forward_argmax");
   hipLaunchKernelGGL(argmax_pairs_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, stream(), ids,
                      pair_val, pair_idx, M, ntn * WGN);
@@ -1325,7 +1364,7 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
 // Ring kernel for small problems: K % 32 == 0.
 template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool PIPE = false>
 static int launch_ring(float* out, const float* inp, const float* weight, const float* bias, int M,
-                       int K, int N, bool gelu, SplitK sk = {}) {
+                       int K, int N, bool gelu, SplitK sk = {}, const float* resid = nullptr) {
   constexpr int NT = WGM * WGN * KS * kWave;
   constexpr size_t lds_bytes = (size_t)NBUF * (BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
@@ -1337,8 +1376,8 @@ static int launch_ring(float* out, const float* inp, const float* weight, const 
     kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true, true, PIPE>
                : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false, true, PIPE>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, M,
-                     K, N, ntm, ntn, sk.ws, sk.cnt, sk.splits);
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, resid,
+                     M, K, N, ntm, ntn, sk.ws, sk.cnt, sk.splits);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1458,42 +1497,42 @@ static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only, size_
 // Launches candidate `best` with the K split of `sk`.
 static int launch_choice(int best, long long best_tiles, float* out, const float* inp, const float* weight,
                          const float* bias, int M, int C, int OC, bool gelu, unsigned long long* probe,
-                         SplitK sk) {
+                         SplitK sk, const float* resid) {
   switch (best) {
     case kTile128x160:
       // four waves of 32x160, two workgroups per compute unit
-      return launch_dma<128, 160, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+      return launch_dma<128, 160, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
     case 8:
       // eight waves of 64x64, one workgroup per compute unit
-      return launch_dma<256, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+      return launch_dma<256, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
     case 7:
       // eight waves of 64x96, one workgroup per compute unit
-      return launch_dma<256, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+      return launch_dma<256, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
     case 6:
       // 64x96: two waves side by side, K split between two such pairs
-      return launch_ring<64, 96, 2, 1, 2, 4, true>(out, inp, weight, bias, M, C, OC, gelu, sk);
+      return launch_ring<64, 96, 2, 1, 2, 4, true>(out, inp, weight, bias, M, C, OC, gelu, sk, resid);
     case 5:
       // one 32x32 tile per workgroup, its four waves splitting K
-      return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu, sk);
+      return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu, sk, resid);
     case 4:
       // up to two workgroups per CU: latency-bound, ring of four slabs and a 2-way K split
       if (best_tiles * sk.splits <= 2 * 256)
-        return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu, sk);
-      return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+        return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu, sk, resid);
+      return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
     case 3:
-      return launch_dma<64, 128, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+      return launch_dma<64, 128, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
     case 2:
       // four waves of 32x96: two workgroups per compute unit
-      return launch_dma<128, 96, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk);
+      return launch_dma<128, 96, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
     case 1:
-      return launch_dma<128, 128, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk);
+      return launch_dma<128, 128, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk, resid);
     default:
       // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
       // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
       // gives every SIMD two waves to alternate between.
       if (best_tiles >= 16 * 256 && sk.splits == 1)
-        return launch_dma<128, 192, 2, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe);
-      return launch_dma<128, 192, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk);
+        return launch_dma<128, 192, 2, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, SplitK{}, resid);
+      return launch_dma<128, 192, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk, resid);
   }
 }
 
@@ -1505,7 +1544,7 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
                            int B, int T, int C, int OC, bool gelu,
                            unsigned long long* probe = nullptr, int* probe_groups = nullptr,
                            void* workspace = nullptr, size_t workspace_bytes = 0,
-                           const ForcedPlan* forced = nullptr) {
+                           const ForcedPlan* forced = nullptr, const float* resid = nullptr) {
   if (B < 0 || T < 0 || C < 1 || OC < 1)
     return fail(GPT2HIP_EINVAL, "matmul_forward: bad shape B=%d T=%d C=%d OC=%d", B, T, C, OC);
   const long long M64 = (long long)B * T;
@@ -1523,12 +1562,12 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
     if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs the MFMA path");
     const size_t total = (size_t)M * OC;
     hipLaunchKernelGGL(matmul_generic_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream(),
-                       out, inp, weight, bias, M, C, OC, gelu ? 1 : 0);
+                       out, inp, weight, bias, resid, M, C, OC, gelu ? 1 : 0);
     G2_LAUNCH_CHECK("matmul_forward");
     return GPT2HIP_OK;
   }
   if (M <= 16 && C % 16 == 0 && !probe && !forced)
-    return skinny_launch(out, inp, weight, bias, nullptr, nullptr, nullptr, M, C, OC, gelu);
+    return skinny_launch(out, inp, weight, bias, nullptr, nullptr, resid, M, C, OC, gelu);
   // per-lane DMA offsets are 32-bit byte offsets inside one tile's rows
   if (tiled) {
     TileChoice choice;
@@ -1552,10 +1591,10 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
       sk.ws = reinterpret_cast<float*>(static_cast<char*>(workspace) + GPT2HIP_SPLITK_COUNTER_BYTES);
       sk.splits = choice.splits;
     }
-    return launch_choice(choice.index, choice.tiles, out, inp, weight, bias, M, C, OC, gelu, probe, sk);
+    return launch_choice(choice.index, choice.tiles, out, inp, weight, bias, M, C, OC, gelu, probe, sk, resid);
   }
   if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs C %% 32 == 0");
-  return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu);
+  return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, resid);
 }
 
 // ---- lm-head + argmax -------------------------------------------------------------------
@@ -1695,6 +1734,19 @@ int matmul_forward_splitk_status(float* out, const float* inp, const float* weig
                                  size_t workspace_bytes) {
   return g2::matmul_dispatch(out, inp, weight, bias, B, T, C, OC, is_gelu != 0, nullptr, nullptr,
                              workspace, workspace_bytes);
+}
+
+int matmul_forward_residual_status(float* out, const float* inp, const float* weight, const float* bias,
+                                   const float* resid, int B, int T, int C, int OC, void* workspace,
+                                   size_t workspace_bytes) {
+  using namespace g2;
+  if (!resid) return fail(GPT2HIP_EINVAL, "matmul_forward_residual: null residual");
+  // the kernels read resid and write out through pointers they are told do not alias
+  const long long n = (long long)(B > 0 ? B : 0) * (T > 0 ? T : 0) * (OC > 0 ? OC : 0);
+  if (out && out < resid + n && resid < out + n)
+    return fail(GPT2HIP_EINVAL, "matmul_forward_residual: out and resid overlap");
+  return matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false, nullptr, nullptr, workspace,
+                         workspace_bytes, nullptr, resid);
 }
 
 int matmul_forward_splitk_forced_status(float* out, const float* inp, const float* weight,

@@ -42,11 +42,14 @@ struct Rng {
 };
 
 int main(int argc, char** argv) {
-  // a small GPT-2: sizes chosen to exercise edge tiles (V and T are not multiples of a tile)
-  const int maxT = 96, V = 1031, L = 3, NH = 4, C = 256, B = 3, T = 77;
+  // a small GPT-2: sizes chosen to exercise edge tiles (V and T are not multiples of a tile).
+  // With the argument "long" the prompts are long enough for the library's own driver to form
+  // the residual sums in the projections' epilogues (gpt2_forward_sums_in_matmul) while this
+  // driver keeps the reference's fused_residual_layernorm_forward: still the same bits.
+  const bool long_prompts = argc > 1 && std::strcmp(argv[1], "long") == 0;
+  const int maxT = long_prompts ? 1024 : 96, V = 1031, L = long_prompts ? 2 : 3, NH = 4, C = 256,
+            B = long_prompts ? 12 : 3, T = long_prompts ? 1021 : 77;
   const size_t c = C;
-  (void)argc;
-  (void)argv;
 
   // parameters in llm.c checkpoint order
   const size_t sizes[16] = {(size_t)V * c, (size_t)maxT * c, L * c,     L * c, L * 3 * c * c, L * 3 * c,
@@ -122,6 +125,10 @@ int main(int argc, char** argv) {
 
   // ---- the library's own driver on the same parameters and tokens ------------------------
   GPT2Config cfg = {maxT, V, L, NH, C};
+  if (gpt2_forward_sums_in_matmul(&cfg, B, T) != (long_prompts ? 1 : 0)) {
+    fprintf(stderr, "gpt2_forward_sums_in_matmul: not the case this run is meant to cover\n");
+    return 2;
+  }
   GPT2* model = gpt2_create(&cfg);
   if (!model || gpt2_load_params_host(model, hp.data(), hp.size()) != GPT2HIP_OK) {
     fprintf(stderr, "gpt2_create / gpt2_load_params_host: %s\n", gpt2hip_last_error());
@@ -144,7 +151,8 @@ int main(int argc, char** argv) {
     maxdiff = std::fmax(maxdiff, std::fabs((double)mine[i] - (double)theirs[i]));
   }
   printf("llmc_style_driver: L=%d C=%d B=%d T=%d V=%d: sum(logits)=%.6f max|launchers - gpt2_forward|=%g "
-         "finite=%d status_form_reports=%d\n", L, C, B, T, V, sum, maxdiff, (int)finite, (int)reports);
+         "finite=%d status_form_reports=%d sums_in_matmul=%d\n", L, C, B, T, V, sum, maxdiff, (int)finite,
+         (int)reports, (int)long_prompts);
 
   gpt2_destroy(model);
   gpt2hip_set_workspace(nullptr, 0);

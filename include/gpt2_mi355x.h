@@ -120,6 +120,17 @@ size_t matmul_forward_splitk_workspace(void);
 int matmul_forward_splitk_status(float* out, const float* inp, const float* weight, const float* bias,
                                  int B, int T, int C, int OC, int is_gelu, void* workspace,
                                  size_t workspace_bytes);
+/* out = resid + (inp . weight^T + bias): the product with a transformer block's residual add in
+ * its epilogue (every workgroup reads the entries of resid that match the tile it is about to
+ * store), so that the add costs no pass of its own over memory.  The reference adds the
+ * residual in the kernel that also normalises (kernels/layernorm/fused_residual_layernorm.cuh:
+ * 88-90, which fused_residual_layernorm_forward keeps as a launcher); the library's gpt2_forward
+ * driver adds it here instead and runs layernorm_forward on the sum: the same additions in the
+ * same order, bit for bit, with half the normalisation kernel's traffic.  resid: (B*T, OC), must
+ * not overlap out.  workspace as for matmul_forward_splitk_status (NULL / 0: none). */
+int matmul_forward_residual_status(float* out, const float* inp, const float* weight, const float* bias,
+                                   const float* resid, int B, int T, int C, int OC, void* workspace,
+                                   size_t workspace_bytes);
 /* The plan matmul_forward_splitk_status would choose: tile shape (0 x 0 for problems outside
  * the tiled kernels) and workgroups per tile (1 = K not split).  Touches no GPU. */
 int matmul_forward_splitk_plan(int B, int T, int C, int OC, size_t workspace_bytes, int* tile_rows,
@@ -295,6 +306,14 @@ int gpt2_decode_probe_status(GPT2* model, const int* next_ids_device, unsigned l
 size_t gpt2_decode_probe_size(const GPT2* model);
 const float* gpt2_step_logits(const GPT2* model);
 int gpt2_cache_length(const GPT2* model);
+
+/* Whether gpt2_forward at this size forms the two residual sums of a block in the epilogues of
+ * the projections (matmul_forward_residual_status, followed by layernorm_forward on the sum)
+ * rather than in fused_residual_layernorm_forward: 1 from B*T*channels = 3 000 000 on, where it
+ * is the faster of the two; the logits are the same bit for bit either way.  In the profiled
+ * pass GPT2_PROF_FUSED_RESIDUAL_LAYERNORM then holds those layernorm_forward launches and the two
+ * projections' categories include the add.  Touches no GPU. */
+int gpt2_forward_sums_in_matmul(const GPT2Config* config, int B, int T);
 
 /* Forward pass that keeps only the argmax of every position's logits (greedy next
  * token ids, B*T ints on the device): the lm-head runs as matmul_forward_argmax, the

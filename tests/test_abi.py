@@ -156,3 +156,15 @@ def test_library_links_no_blas():
     syms = subprocess.run(["nm", "-D", "--undefined-only", g2.LIB_PATH], capture_output=True, text=True,
                           check=True).stdout
     assert not re.search(r"rocblas_|hipblas|hipblaslt", syms, re.I)
+
+
+def test_where_the_driver_forms_the_residual_sums_is_a_pure_function_of_the_size():
+    """gpt2_forward adds the residual stream in the projections' epilogues from B*T*channels =
+    3e6 on (the headline size and GPT-2 350M at B=4) and keeps the reference's fused
+    residual+layernorm below; the answer needs no GPU."""
+    assert g2.forward_sums_in_matmul(g2.GPT2_124M, 8, 1024)
+    assert g2.forward_sums_in_matmul(g2.GPT2_124M, 4, 1024)
+    assert g2.forward_sums_in_matmul(g2.GPT2_350M, 4, 1024)
+    assert not g2.forward_sums_in_matmul(g2.GPT2_124M, 2, 1024)
+    assert not g2.forward_sums_in_matmul(g2.GPT2_124M, 4, 64)
+    assert g2.lib().gpt2_forward_sums_in_matmul(None, 8, 1024) == 0

@@ -563,11 +563,15 @@ def test_cpp_driver_calling_the_launchers_equals_gpt2_forward():
     for bit, and the _status forms must report errors instead of aborting."""
     import subprocess
     assert os.path.exists(g2.EXAMPLE_BIN), "build() compiles the example driver"
-    print("running", g2.EXAMPLE_BIN, flush=True)
-    proc = subprocess.run([g2.EXAMPLE_BIN], capture_output=True, text=True, timeout=100)
-    print(proc.stdout, proc.stderr, flush=True)
-    assert proc.returncode == 0
-    assert "max|launchers - gpt2_forward|=0 " in proc.stdout
+    # second run: prompts long enough for gpt2_forward to add the residual stream in the
+    # projections' epilogues, while the example keeps fused_residual_layernorm_forward
+    for extra in ([], ["long"]):
+        print("running", g2.EXAMPLE_BIN, *extra, flush=True)
+        proc = subprocess.run([g2.EXAMPLE_BIN, *extra], capture_output=True, text=True, timeout=100)
+        print(proc.stdout, proc.stderr, flush=True)
+        assert proc.returncode == 0
+        assert "max|launchers - gpt2_forward|=0 " in proc.stdout
+        assert f"sums_in_matmul={len(extra)}" in proc.stdout
 
 
 def test_gpt2_decode_error_paths():

@@ -353,6 +353,52 @@ def test_matmul_llmc_signature_splits_k_through_the_thread_workspace(M, splitk_w
     assert torch.equal(again, plain)
 
 
+# out = resid + (x . w^T + b), the residual add in the product's epilogue: every kernel family
+# (the LDS-DMA kernel with the tile of resid fetched during the slab loop at 128x192 / 128x128 /
+# 128x96, the same kernel reading it in the epilogue at 256x192, the ring kernel, K split between
+# workgroups, edge tiles, the <= 16-row kernel, the generic one).  The sum must equal the plain
+# product plus resid bit for bit (one fp32 addition per entry, the product's bits unchanged).
+@pytest.mark.parametrize("M,C,OC", [
+    (8192, 768, 768), (8192, 3072, 768), (4096, 1024, 1024), (4090, 768, 770), (8192, 768, 3072),
+    (6000, 768, 1536), (4096, 1280, 1280), (2048, 768, 768), (2045, 3072, 771), (256, 3072, 768),
+    (100, 96, 50), (33, 30, 17), (8, 768, 768)])
+@pytest.mark.parametrize("lend", [False, True])
+def test_matmul_residual_epilogue(M, C, OC, lend, splitk_workspace):
+    ws = splitk_workspace if lend else None
+    plan = g2.matmul_forward_splitk_plan(1, M, C, OC, ws.numel() if lend else 0)
+    say(f"matmul + residual M={M} C={C} OC={OC} workspace={lend} plan={plan}")
+    x, w, b = mm_inputs(M, C, OC, 135)
+    r = np.random.default_rng(136).standard_normal((M, OC), dtype=np.float32)
+    dx, dw, db, dr = dev(x), dev(w), dev(b), dev(r)
+    plain = torch.empty((M, OC), device="cuda")
+    g2.matmul_forward_splitk(plain, dx, dw, db, 1, M, C, OC, ws)
+    full, out, pad = guard((M, OC))
+    g2.matmul_forward_residual(out, dx, dw, db, dr, 1, M, C, OC, ws)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    assert torch.equal(dr, dev(r)), "resid was modified"
+    assert torch.equal(out, plain + dr), "not the plain product plus resid"
+    if lend:
+        assert int(ws[:g2.SPLITK_COUNTER_BYTES].max()) == 0, "counters not left at zero"
+    elif M * C * OC <= 8192 * 768 * 768:
+        assert_close(out, oracle.matmul_forward(x, w, b) + r, "matmul + residual")
+
+
+def test_matmul_residual_rejects_overlap_and_null():
+    M, C, OC = 64, 64, 64
+    x, w, b = mm_inputs(M, C, OC, 137)
+    buf = torch.zeros(2 * M * OC, device="cuda")
+    out = buf[:M * OC].view(M, OC)
+    with pytest.raises(RuntimeError, match="overlap"):
+        g2.matmul_forward_residual(out, dev(x), dev(w), dev(b), out, 1, M, C, OC)
+    with pytest.raises(RuntimeError, match="overlap"):
+        g2.matmul_forward_residual(out, dev(x), dev(w), dev(b), buf[OC:OC + M * OC].view(M, OC), 1, M, C, OC)
+    with pytest.raises(RuntimeError, match="null residual"):
+        g2.matmul_forward_residual(out, dev(x), dev(w), dev(b), None, 1, M, C, OC)
+    g2.matmul_forward_residual(out, dev(x), dev(w), dev(b), buf[M * OC:].view(M, OC), 1, M, C, OC)
+    torch.cuda.synchronize()
+
+
 def test_matmul_splitk_rejects_what_does_not_fit(splitk_workspace):
     x, w, b = mm_inputs(64, 64, 64, 133)
     out = torch.empty((64, 64), device="cuda")
