@@ -43,7 +43,7 @@ EXPORTS = (
     "matmul_forward_tile_shape",
     "matmul_forward_splitk_workspace", "matmul_forward_splitk_status",
     "matmul_forward_splitk_plan", "matmul_forward_splitk_forced_status",
-    "matmul_forward_residual_status",
+    "matmul_forward_residual_status", "matmul_forward_first_columns",
     "attention_forward", "attention_forward_status",
     "argmax_forward", "argmax_forward_status",
     "matmul_forward_argmax_workspace", "matmul_forward_argmax_status",
@@ -145,6 +145,8 @@ def lib() -> ctypes.CDLL:
         L.matmul_forward_splitk_status.restype = ci
         L.matmul_forward_splitk_forced_status.argtypes = [vp] * 4 + [ci] * 5 + [vp, cz] + [ci] * 3
         L.matmul_forward_splitk_forced_status.restype = ci
+        L.matmul_forward_first_columns.argtypes = [ci] * 4 + [cz]
+        L.matmul_forward_first_columns.restype = ci
         L.matmul_forward_residual_status.argtypes = [vp] * 5 + [ci] * 4 + [vp, cz]
         L.matmul_forward_residual_status.restype = ci
         L.matmul_forward_splitk_plan.argtypes = [ci] * 4 + [cz] + [ctypes.POINTER(ci)] * 3
@@ -327,6 +329,11 @@ def matmul_forward_residual(out, inp, weight, bias, resid, B, T, C, OC, workspac
     _check(lib().matmul_forward_residual_status(_f32(out), _f32(inp), _f32(weight), _f32(bias),
                                                 _f32(resid), B, T, C, OC, ws, nbytes),
            "matmul_forward_residual")
+
+
+def matmul_forward_first_columns(B, T, C, OC, workspace_bytes=0):
+    """Columns computed by the first launch of a product (OC: the product is one launch)."""
+    return lib().matmul_forward_first_columns(B, T, C, OC, workspace_bytes)
 
 
 def forward_sums_in_matmul(config, B, T):

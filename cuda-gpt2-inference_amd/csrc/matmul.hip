@@ -123,46 +123,47 @@ __device__ __forceinline__ void argmax_fold(float* bv, int* bx, int lane, int& f
 // GELU if asked), plus resid's entries of the same positions where resid is given (the residual
 // add of a transformer block, which then needs no pass of its own over memory: out = resid +
 // act(product); out and resid must not overlap).  row0 / col0: this lane's first row and its
-// column in the wave's first tile.  All of a wave's loads of resid are issued before its first
-// store.
+// column in the wave's first tile; ldo: floats from one row of out (and of resid) to the next,
+// N unless the launch computes a range of the columns of a wider product.  All of a wave's loads
+// of resid are issued before its first store.
 // (a full tile's entries of resid, in the accumulators' layout)
 template <int TM, int TN>
 __device__ __forceinline__ void load_resid_tile(f32x16 (&rs)[TM][TN], const float* __restrict__ resid,
-                                                int row0, int col0, int N) {
+                                                int row0, int col0, int ldo) {
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const float* const rp = resid + (size_t)(row0 + i * 32) * N + col0 + j * 32;
+      const float* const rp = resid + (size_t)(row0 + i * 32) * ldo + col0 + j * 32;
 #pragma unroll
-      for (int v = 0; v < 16; v++) rs[i][j][v] = rp[(size_t)(8 * (v >> 2) + (v & 3)) * N];
+      for (int v = 0; v < 16; v++) rs[i][j][v] = rp[(size_t)(8 * (v >> 2) + (v & 3)) * ldo];
     }
 }
 // (a full tile: out = act(acc) + rs)
 template <int TM, int TN, bool GELU>
 __device__ __forceinline__ void store_tile_sum(const f32x16 (&acc)[TM][TN], const f32x16 (&rs)[TM][TN],
-                                               float* __restrict__ out, int row0, int col0, int N) {
+                                               float* __restrict__ out, int row0, int col0, int ldo) {
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      float* const o = out + (size_t)(row0 + i * 32) * N + col0 + j * 32;
+      float* const o = out + (size_t)(row0 + i * 32) * ldo + col0 + j * 32;
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         float r = acc[i][j][v];
         if (GELU) r = gelu_tanh(r);
-        o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r + rs[i][j][v];
+        o[(size_t)(8 * (v >> 2) + (v & 3)) * ldo] = r + rs[i][j][v];
       }
     }
 }
 template <int TM, int TN, bool GELU>
 __device__ __forceinline__ void store_tile(const f32x16 (&acc)[TM][TN], float* __restrict__ out,
                                            const float* __restrict__ resid, int row0, int col0, int M,
-                                           int N, bool full) {
+                                           int N, int ldo, bool full) {
   if (full && resid != nullptr) {
     f32x16 rs[TM][TN];
-    load_resid_tile<TM, TN>(rs, resid, row0, col0, N);
-    store_tile_sum<TM, TN, GELU>(acc, rs, out, row0, col0, N);
+    load_resid_tile<TM, TN>(rs, resid, row0, col0, ldo);
+    store_tile_sum<TM, TN, GELU>(acc, rs, out, row0, col0, ldo);
     return;
   }
 #pragma unroll
@@ -171,13 +172,13 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[TM][TN], float* _
     for (int j = 0; j < TN; j++) {
       const int col = col0 + j * 32;
       const int rbase = row0 + i * 32;
-      float* o = out + (size_t)rbase * N + col;
+      float* o = out + (size_t)rbase * ldo + col;
       if (full) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           float r = acc[i][j][v];
           if (GELU) r = gelu_tanh(r);
-          o[(size_t)(8 * (v >> 2) + (v & 3)) * N] = r;
+          o[(size_t)(8 * (v >> 2) + (v & 3)) * ldo] = r;
         }
       } else if (col < N) {
 #pragma unroll
@@ -186,8 +187,8 @@ __device__ __forceinline__ void store_tile(const f32x16 (&acc)[TM][TN], float* _
           if (row < M) {
             float r = acc[i][j][v];
             if (GELU) r = gelu_tanh(r);
-            if (resid != nullptr) r += resid[(size_t)row * N + col];
-            out[(size_t)row * N + col] = r;
+            if (resid != nullptr) r += resid[(size_t)row * ldo + col];
+            out[(size_t)row * ldo + col] = r;
           }
         }
       }
@@ -267,7 +268,8 @@ __device__ __forceinline__ bool splitk_combine(f32x16 (&acc)[TM][TN], float* __r
 template <int BM, int BN, int WGM, int WGN, bool GELU, bool KTAIL>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ntm, int ntn) {
+    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ldo, int ntm,
+    int ntn) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -452,7 +454,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_mfma_kernel(
 
   // ---- epilogue -----------------------------------------------------------
   const bool full = (m0 + BM <= M) && (n0 + BN <= N);
-  store_tile<TM, TN, GELU>(acc, out, resid, m0 + wm * WM + 4 * h, n0 + wn * WN + (lane & 31), M, N, full);
+  store_tile<TM, TN, GELU>(acc, out, resid, m0 + wm * WM + 4 * h, n0 + wn * WN + (lane & 31), M, N, ldo, full);
 }
 
 // ---------------------------------------------------------------------------
@@ -495,8 +497,8 @@ template <int BM, int BN, int WGM, int WGN, bool GELU, bool PROBE = false, bool 
           bool SPLIT = false, bool RESID = false>
 __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ntm, int ntn,
-    unsigned long long* __restrict__ probe, int* __restrict__ arg_idx, float* __restrict__ part_ws,
+    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ldo, int ntm,
+    int ntn, unsigned long long* __restrict__ probe, int* __restrict__ arg_idx, float* __restrict__ part_ws,
     unsigned* __restrict__ part_cnt, int splits) {
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -688,7 +690,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   if constexpr (RESID) {
     for (; s + 1 < nslab; s += 2) {
       if ((s >> 1) == resid_at) {
-        load_resid_tile<TM, TN>(rs, resid, row0, col0, N);
+        load_resid_tile<TM, TN>(rs, resid, row0, col0, ldo);
         resid_loaded = true;
       }
       slab_body(s, std::integral_constant<int, 0>{});
@@ -697,7 +699,7 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   }
   if (s < nslab) slab_body(s, std::integral_constant<int, 0>{});
   if constexpr (RESID) {
-    if (full && !resid_loaded) load_resid_tile<TM, TN>(rs, resid, row0, col0, N);
+    if (full && !resid_loaded) load_resid_tile<TM, TN>(rs, resid, row0, col0, ldo);
   }
   if (PROBE && tid == 0) {
     probe[4 * blockIdx.x + 0] = wall0;
@@ -760,14 +762,14 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
   }
   if constexpr (RESID) {
     if (full) {
-      store_tile_sum<TM, TN, GELU>(acc, rs, out, row0, col0, N);
+      store_tile_sum<TM, TN, GELU>(acc, rs, out, row0, col0, ldo);
       return;
     }
   }
   // A product larger than the 256 MiB Infinity Cache (the logits) will not be read back
   // from any cache: its tiles are stored with streaming stores, so that they do not push
   // the operands that other tiles are about to re-read out of L2.
-  const bool stream_out = (size_t)M * N * sizeof(float) > ((size_t)256 << 20);
+  const bool stream_out = (size_t)M * ldo * sizeof(float) > ((size_t)256 << 20);
   if (full && stream_out && resid == nullptr) {
     // Row by row: the wave's TN segments of 128 bytes of one row go out back to back, as one run
     // of TN * 128 bytes.  Rows of such a product (N = 50257) start at any multiple of 4 bytes, so
@@ -775,20 +777,20 @@ __global__ __launch_bounds__(WGM* WGN* kWave) void matmul_dma_kernel(
     // merged there, and only the two ends of the run are left as partial lines.
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-      float* const o = out + (size_t)(m0 + wm * WM + i * 32 + 4 * h) * N + n0 + wn * WN + (lane & 31);
+      float* const o = out + (size_t)(m0 + wm * WM + i * 32 + 4 * h) * ldo + n0 + wn * WN + (lane & 31);
 #pragma unroll
       for (int v = 0; v < 16; v++) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
           float r = acc[i][j][v];
           if (GELU) r = gelu_tanh(r);
-          __builtin_nontemporal_store(r, o + (size_t)(8 * (v >> 2) + (v & 3)) * N + j * 32);
+          __builtin_nontemporal_store(r, o + (size_t)(8 * (v >> 2) + (v & 3)) * ldo + j * 32);
         }
       }
     }
     return;
   }
-  store_tile<TM, TN, GELU>(acc, out, resid, row0, col0, M, N, full);
+  store_tile<TM, TN, GELU>(acc, out, resid, row0, col0, M, N, ldo, full);
 }
 
 // s_waitcnt immediate that waits until at most n vector-memory operations of this wave
@@ -814,8 +816,8 @@ template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool GELU, bool SP
           bool PIPE = false>
 __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
     float* __restrict__ out, const float* __restrict__ inp, const float* __restrict__ weight,
-    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ntm, int ntn,
-    float* __restrict__ part_ws, unsigned* __restrict__ part_cnt, int splits) {
+    const float* __restrict__ bias, const float* __restrict__ resid, int M, int K, int N, int ldo, int ntm,
+    int ntn, float* __restrict__ part_ws, unsigned* __restrict__ part_cnt, int splits) {
   constexpr int NMN = WGM * WGN;
   constexpr int NW = NMN * KS;
   constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -1044,7 +1046,7 @@ __global__ __launch_bounds__(WGM* WGN* KS* kWave) void matmul_ring_kernel(
   }
 
   const bool full = (m0 + BM <= M) && (n0 + BN <= N);
-  store_tile<TM, TN, GELU>(acc, out, resid, m0 + wm * WM + 4 * h, n0 + wn * WN + (lane & 31), M, N, full);
+  store_tile<TM, TN, GELU>(acc, out, resid, m0 + wm * WM + 4 * h, n0 + wn * WN + (lane & 31), M, N, ldo, full);
 }
 
 // M <= 16 rows (one token per sequence: a decode step).  Such a product is bound by
@@ -1279,10 +1281,18 @@ static int allow_lds(const void* kfn, size_t lds_bytes) {
   return GPT2HIP_OK;
 }
 
+// What a launch does beyond out = act(inp . weight^T + bias).  resid (optional): added in the
+// epilogue.  ldo (0: N): floats from one row of out (and of resid) to the next, when the launch
+// computes a range of the columns of a wider product.
+struct Epilogue {
+  const float* resid = nullptr;
+  int ldo = 0;
+};
+
 // Register-staged kernel: any K % 4 == 0.
 template <int BM, int BN, int WGM, int WGN>
 static int launch_mfma(float* out, const float* inp, const float* weight, const float* bias, int M,
-                       int K, int N, bool gelu, const float* resid = nullptr) {
+                       int K, int N, bool gelu, Epilogue epi = {}) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
@@ -1294,8 +1304,8 @@ static int launch_mfma(float* out, const float* inp, const float* weight, const 
                    : (gelu ? matmul_mfma_kernel<BM, BN, WGM, WGN, true, false>
                            : matmul_mfma_kernel<BM, BN, WGM, WGN, false, false>);
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, resid,
-                     M, K, N, ntm, ntn);
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias,
+                     epi.resid, M, K, N, epi.ldo ? epi.ldo : N, ntm, ntn);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1312,7 +1322,7 @@ struct SplitK {
 template <int BM, int BN, int WGM, int WGN, bool PROBED = false>
 static int launch_dma(float* out, const float* inp, const float* weight, const float* bias, int M,
                       int K, int N, bool gelu, unsigned long long* probe = nullptr, SplitK sk = {},
-                      const float* resid = nullptr) {
+                      Epilogue epi = {}) {
   constexpr int NT = WGM * WGN * kWave;
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
@@ -1323,7 +1333,7 @@ static int launch_dma(float* out, const float* inp, const float* weight, const f
     if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: no probe form with K split");
     kfn = gelu ? matmul_dma_kernel<BM, BN, WGM, WGN, true, false, false, true>
                : matmul_dma_kernel<BM, BN, WGM, WGN, false, false, false, true>;
-  } else if (resid && !gelu && !probe && (BM / WGM / 32) * (BN / WGN / 32) <= 3) {
+  } else if (epi.resid && !gelu && !probe && (BM / WGM / 32) * (BN / WGN / 32) <= 3) {
     // (larger register tiles have no room for the tile of resid beside the accumulators: they read
     // it in the epilogue)
     if constexpr ((BM / WGM / 32) * (BN / WGN / 32) <= 3)
@@ -1334,8 +1344,9 @@ static int launch_dma(float* out, const float* inp, const float* weight, const f
     return fail(GPT2HIP_EINVAL, "matmul_forward_probe: no probe form of the %dx%d tile", BM, BN);
   }
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, resid,
-                     M, K, N, ntm, ntn, probe, (int*)nullptr, sk.ws, sk.cnt, sk.splits);
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias,
+                     epi.resid, M, K, N, epi.ldo ? epi.ldo : N, ntm, ntn, probe, (int*)nullptr, sk.ws, sk.cnt,
+                     sk.splits);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1352,7 +1363,7 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
   auto kfn = matmul_dma_kernel<BM, BN, WGM, WGN, false, false, true>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
   hipLaunchKernelGGL(kfn, dim3((unsigned)(ntm * ntn)), dim3(NT), lds_bytes, stream(), pair_val, inp, weight,
-                     bias, (const float*)nullptr, M, K, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx,
+                     bias, (const float*)nullptr, M, K, N, N, ntm, ntn, (unsigned long long*)nullptr, pair_idx,
                      (float*)nullptr, (unsigned*)nullptr, 1);
   G2_LAUNCH_CHECK("matmul_forward_argmax");
   hipLaunchKernelGGL(argmax_pairs_kernel, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, stream(), ids,
@@ -1364,7 +1375,7 @@ static int launch_dma_argmax(int* ids, float* pair_val, int* pair_idx, const flo
 // Ring kernel for small problems: K % 32 == 0.
 template <int BM, int BN, int WGM, int WGN, int KS, int NBUF, bool PIPE = false>
 static int launch_ring(float* out, const float* inp, const float* weight, const float* bias, int M,
-                       int K, int N, bool gelu, SplitK sk = {}, const float* resid = nullptr) {
+                       int K, int N, bool gelu, SplitK sk = {}, Epilogue epi = {}) {
   constexpr int NT = WGM * WGN * KS * kWave;
   constexpr size_t lds_bytes = (size_t)NBUF * (BM + BN) * BK * sizeof(float);
   const int ntm = (M + BM - 1) / BM, ntn = (N + BN - 1) / BN;
@@ -1376,8 +1387,8 @@ static int launch_ring(float* out, const float* inp, const float* weight, const 
     kfn = gelu ? matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, true, true, PIPE>
                : matmul_ring_kernel<BM, BN, WGM, WGN, KS, NBUF, false, true, PIPE>;
   if (int rc = allow_lds(reinterpret_cast<const void*>(kfn), lds_bytes)) return rc;
-  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias, resid,
-                     M, K, N, ntm, ntn, sk.ws, sk.cnt, sk.splits);
+  hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(NT), lds_bytes, stream(), out, inp, weight, bias,
+                     epi.resid, M, K, N, epi.ldo ? epi.ldo : N, ntm, ntn, sk.ws, sk.cnt, sk.splits);
   G2_LAUNCH_CHECK("matmul_forward");
   return GPT2HIP_OK;
 }
@@ -1399,6 +1410,7 @@ struct TileChoice {
   int bm, bn;
   long long tiles;
   int splits;       // workgroups per tile (K split between them), 1 = none
+  double cost_us;   // what the model below expects the launch to take
 };
 // fix_*: what a K split between workgroups adds (fitted per shape to a second forced sweep, over
 // 2..8 parts): fix_us + fix_part_us x parts + fix_mb_us x MB of partial tiles.  The partial
@@ -1445,6 +1457,23 @@ static bool split_fits(int i, int M, int C, int OC, int splits, size_t workspace
   return need <= workspace_bytes - GPT2HIP_SPLITK_COUNTER_BYTES;
 }
 
+// The constants of candidate i as it is launched for `groups` workgroups, and the model's time for
+// t tiles of it with K split S ways (without what the split itself adds).
+static TileCand cand_form(int i, long long groups) {
+  TileCand k = kTileCands[i];
+  if (i == 4 && groups <= 2 * 256) {  // the ring form of 64x64
+    k.a = 1.190;
+    k.round_us = 0.35;
+    k.launch_us = 2.98;
+  }
+  return k;
+}
+static double tile_cost(int i, long long t, int C, int S) {
+  const TileCand k = cand_form(i, t * S);
+  const double work_us = 2.0 * k.bm * k.bn * (double)C / kCuFlopsPerUs;
+  return k.launch_us + (double)((t * S + 255) / 256) * (k.a * work_us / S + k.round_us);
+}
+
 // workspace_bytes == 0: no K split between workgroups.
 static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only, size_t workspace_bytes = 0) {
   int best = 0, split_best = -1, split_parts = 1;
@@ -1455,21 +1484,14 @@ static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only, size_
     // 128x192 or 320 of 128x128); the GPT-2 124M / 350M widths are no multiples of 160
     if (i == kTile128x160 && OC % 160 != 0) continue;
     const long long t = tiles_of(i, M, OC);
-    TileCand c = kTileCands[i];
-    const double work_us = 2.0 * c.bm * c.bn * (double)C / kCuFlopsPerUs;
     // K split S ways: S times the workgroups, each with 1/S of the matrix work, plus the
     // partial tiles' trip through memory (written once, read once by the last arrival)
     for (int S = 1; S <= 8; S++) {
       if (S > 1 && (workspace_bytes == 0 || two_largest_only || t * S > 6 * 256 ||
                     !split_fits(i, M, C, OC, S, workspace_bytes)))
         continue;
-      TileCand k = c;
-      if (i == 4 && t * S <= 2 * 256) {  // the ring form of 64x64
-        k.a = 1.190;
-        k.round_us = 0.35;
-        k.launch_us = 2.98;
-      }
-      double cost = k.launch_us + (double)((t * S + 255) / 256) * (k.a * work_us / S + k.round_us);
+      const TileCand k = cand_form(i, t * S);
+      double cost = tile_cost(i, t, C, S);
       if (S == 1) {
         if (i == 0 || cost < best_cost) {
           best = i;
@@ -1490,49 +1512,89 @@ static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only, size_
   }
   if (split_best >= 0 && split_cost * kSplitMargin < best_cost)
     return TileChoice{split_best, kTileCands[split_best].bm, kTileCands[split_best].bn,
-                      tiles_of(split_best, M, OC), split_parts};
-  return TileChoice{best, kTileCands[best].bm, kTileCands[best].bn, tiles_of(best, M, OC), 1};
+                      tiles_of(split_best, M, OC), split_parts, split_cost};
+  return TileChoice{best, kTileCands[best].bm, kTileCands[best].bn, tiles_of(best, M, OC), 1, best_cost};
+}
+
+// A product much wider than tall whose tiles come out just above a whole number of rounds loses
+// most of a round to the few tiles left over: the lm-head's 50257 columns are 261.75 tiles of
+// 192, so at 256 rows there are 262 tiles of 256x192 for 256 compute units, and at 1024 rows
+// 4 x 262.  Such a product is computed by two launches over ranges of its columns instead: a
+// whole number of rounds of the tile that suits it, then the few columns left with whatever
+// suits those (measured for the 768 -> 50257 lm-head: 216 -> 180 us at 256 rows, 348 -> 324 at
+// 512, 619 -> 590 at 1024, 1150 -> 1136 at 2048; within 0.5 % either way from 4096 rows on, where
+// the product is left as one launch).
+struct ColumnPlan {
+  int main_cols;         // columns of the first launch; == OC: one launch
+  TileChoice main, rest;
+};
+static ColumnPlan plan_columns(int M, int C, int OC, bool two_largest_only, size_t workspace_bytes) {
+  ColumnPlan plan{OC, choose_tile(M, C, OC, two_largest_only, workspace_bytes), TileChoice{}};
+  if (two_largest_only || OC < 8192) return plan;
+  double best = plan.main.cost_us * 0.97;  // a second launch has to pay for itself
+  static const int kWide[] = {0, 7, 1, 8};  // 128x192, 256x192, 128x128, 256x128
+  for (int i : kWide) {
+    const long long ntm = (M + kTileCands[i].bm - 1) / kTileCands[i].bm;
+    const int ntn_all = OC / kTileCands[i].bn;
+    for (int ntn = ntn_all; ntn >= 1 && ntn > ntn_all - 16; ntn--) {
+      const long long t = ntm * ntn;
+      if (t % 256 != 0) continue;
+      if (t > 12 * 256) break;  // the more rounds, the less the last one matters
+      const int cols = ntn * kTileCands[i].bn;
+      if (cols == OC) break;  // (whole rounds already)
+      const TileChoice rest = choose_tile(M, C, OC - cols, false, workspace_bytes);
+      const double cost = tile_cost(i, t, C, 1) + rest.cost_us;
+      if (cost < best) {
+        best = cost;
+        plan.main_cols = cols;
+        plan.main = TileChoice{i, kTileCands[i].bm, kTileCands[i].bn, t, 1, tile_cost(i, t, C, 1)};
+        plan.rest = rest;
+      }
+      break;  // the widest whole number of rounds of this tile
+    }
+  }
+  return plan;
 }
 
 // Launches candidate `best` with the K split of `sk`.
 static int launch_choice(int best, long long best_tiles, float* out, const float* inp, const float* weight,
                          const float* bias, int M, int C, int OC, bool gelu, unsigned long long* probe,
-                         SplitK sk, const float* resid) {
+                         SplitK sk, Epilogue epi) {
   switch (best) {
     case kTile128x160:
       // four waves of 32x160, two workgroups per compute unit
-      return launch_dma<128, 160, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
+      return launch_dma<128, 160, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, epi);
     case 8:
       // eight waves of 64x64, one workgroup per compute unit
-      return launch_dma<256, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
+      return launch_dma<256, 128, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, epi);
     case 7:
       // eight waves of 64x96, one workgroup per compute unit
-      return launch_dma<256, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
+      return launch_dma<256, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, epi);
     case 6:
       // 64x96: two waves side by side, K split between two such pairs
-      return launch_ring<64, 96, 2, 1, 2, 4, true>(out, inp, weight, bias, M, C, OC, gelu, sk, resid);
+      return launch_ring<64, 96, 2, 1, 2, 4, true>(out, inp, weight, bias, M, C, OC, gelu, sk, epi);
     case 5:
       // one 32x32 tile per workgroup, its four waves splitting K
-      return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu, sk, resid);
+      return launch_ring<32, 32, 1, 1, 4, 4>(out, inp, weight, bias, M, C, OC, gelu, sk, epi);
     case 4:
       // up to two workgroups per CU: latency-bound, ring of four slabs and a 2-way K split
       if (best_tiles * sk.splits <= 2 * 256)
-        return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu, sk, resid);
-      return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
+        return launch_ring<64, 64, 2, 2, 2, 4>(out, inp, weight, bias, M, C, OC, gelu, sk, epi);
+      return launch_dma<64, 64, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, epi);
     case 3:
-      return launch_dma<64, 128, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
+      return launch_dma<64, 128, 2, 2>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, epi);
     case 2:
       // four waves of 32x96: two workgroups per compute unit
-      return launch_dma<128, 96, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, resid);
+      return launch_dma<128, 96, 4, 1>(out, inp, weight, bias, M, C, OC, gelu, nullptr, sk, epi);
     case 1:
-      return launch_dma<128, 128, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk, resid);
+      return launch_dma<128, 128, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk, epi);
     default:
       // Many tiles per CU: 4 waves with 64x96 register tiles, two workgroups per CU.
       // Few tiles per CU: 8 waves with 32x96 tiles, so that a lone workgroup still
       // gives every SIMD two waves to alternate between.
       if (best_tiles >= 16 * 256 && sk.splits == 1)
-        return launch_dma<128, 192, 2, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, SplitK{}, resid);
-      return launch_dma<128, 192, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk, resid);
+        return launch_dma<128, 192, 2, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, SplitK{}, epi);
+      return launch_dma<128, 192, 4, 2, true>(out, inp, weight, bias, M, C, OC, gelu, probe, sk, epi);
   }
 }
 
@@ -1581,7 +1643,23 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
                     forced->splits, forced->bm, forced->bn, C / BK, workspace_bytes);
       choice = TileChoice{idx, forced->bm, forced->bn, tiles_of(idx, M, OC), forced->splits};
     } else {
-      choice = choose_tile(M, C, OC, probe != nullptr, workspace_bytes);
+      const ColumnPlan cp = plan_columns(M, C, OC, probe != nullptr, workspace_bytes);
+      choice = cp.main;
+      if (cp.main_cols != OC) {
+        // two launches over ranges of the columns; rows of out (and resid) stay OC floats apart
+        const size_t n1 = (size_t)cp.main_cols;
+        if (int rc = launch_choice(cp.main.index, cp.main.tiles, out, inp, weight, bias, M, C, cp.main_cols, gelu,
+                                   nullptr, SplitK{}, Epilogue{resid, OC}))
+          return rc;
+        SplitK sk;
+        if (cp.rest.splits > 1) {
+          sk.cnt = static_cast<unsigned*>(workspace);
+          sk.ws = reinterpret_cast<float*>(static_cast<char*>(workspace) + GPT2HIP_SPLITK_COUNTER_BYTES);
+          sk.splits = cp.rest.splits;
+        }
+        return launch_choice(cp.rest.index, cp.rest.tiles, out + n1, inp, weight + n1 * C, bias ? bias + n1 : nullptr,
+                             M, C, OC - cp.main_cols, gelu, nullptr, sk, Epilogue{resid ? resid + n1 : nullptr, OC});
+      }
     }
     if (choice.tiles * choice.splits > 0x7fffffffLL) return fail(GPT2HIP_EINVAL, "matmul_forward: too many tiles");
     if (probe_groups) *probe_groups = (int)choice.tiles;
@@ -1591,10 +1669,11 @@ static int matmul_dispatch(float* out, const float* inp, const float* weight, co
       sk.ws = reinterpret_cast<float*>(static_cast<char*>(workspace) + GPT2HIP_SPLITK_COUNTER_BYTES);
       sk.splits = choice.splits;
     }
-    return launch_choice(choice.index, choice.tiles, out, inp, weight, bias, M, C, OC, gelu, probe, sk, resid);
+    return launch_choice(choice.index, choice.tiles, out, inp, weight, bias, M, C, OC, gelu, probe, sk,
+                         Epilogue{resid, 0});
   }
   if (probe) return fail(GPT2HIP_EINVAL, "matmul_forward_probe: needs C %% 32 == 0");
-  return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, resid);
+  return launch_mfma<128, 192, 4, 2>(out, inp, weight, bias, M, C, OC, gelu, Epilogue{resid, 0});
 }
 
 // ---- lm-head + argmax -------------------------------------------------------------------
@@ -1692,7 +1771,7 @@ int matmul_forward_tile_shape(int B, int T, int C, int OC, int* tile_rows, int* 
     *tile_rows = *tile_cols = 0;  // not one of the tiled LDS-DMA kernels
     return GPT2HIP_OK;
   }
-  const TileChoice c = choose_tile((int)M64, C, OC, false);
+  const TileChoice c = plan_columns((int)M64, C, OC, false, 0).main;
   *tile_rows = c.bm;
   *tile_cols = c.bn;
   return GPT2HIP_OK;
@@ -1769,11 +1848,19 @@ int matmul_forward_splitk_plan(int B, int T, int C, int OC, size_t workspace_byt
     *splits = 1;
     return GPT2HIP_OK;
   }
-  const TileChoice c = choose_tile((int)M64, C, OC, false, workspace_bytes);
+  const TileChoice c = plan_columns((int)M64, C, OC, false, workspace_bytes).main;
   *tile_rows = c.bm;
   *tile_cols = c.bn;
   *splits = c.splits;
   return GPT2HIP_OK;
+}
+
+int matmul_forward_first_columns(int B, int T, int C, int OC, size_t workspace_bytes) {
+  using namespace g2;
+  const long long M64 = (long long)B * T;
+  if (B < 1 || T < 1 || C < 1 || OC < 1 || M64 > 0x7fffffffLL) return 0;
+  if (C % BK != 0 || M64 <= 16 || (long long)C * 192 * 4 >= (1LL << 31)) return OC;
+  return plan_columns((int)M64, C, OC, false, workspace_bytes).main_cols;
 }
 
 int matmul_forward_gelu_status(float* out, const float* inp, const float* weight,

@@ -168,3 +168,16 @@ def test_where_the_driver_forms_the_residual_sums_is_a_pure_function_of_the_size
     assert not g2.forward_sums_in_matmul(g2.GPT2_124M, 2, 1024)
     assert not g2.forward_sums_in_matmul(g2.GPT2_124M, 4, 64)
     assert g2.lib().gpt2_forward_sums_in_matmul(None, 8, 1024) == 0
+
+
+def test_wide_products_are_planned_as_whole_rounds_plus_the_columns_left():
+    """The lm-head at a few hundred to a few thousand rows: the first launch covers a whole
+    number of rounds of its tile over the 256 compute units; tall or narrow products are one launch."""
+    for M in (256, 512, 1024, 2048):
+        first = g2.matmul_forward_first_columns(1, M, 768, 50257)
+        bm, bn = g2.matmul_forward_tile_shape(1, M, 768, 50257)
+        assert 0 < first < 50257 and first % bn == 0 and (first // bn) * -(-M // bm) % 256 == 0, (M, first, bm, bn)
+    assert g2.matmul_forward_first_columns(1, 8192, 768, 50257) == 50257
+    assert g2.matmul_forward_first_columns(1, 2048, 768, 3072) == 3072
+    assert g2.matmul_forward_first_columns(1, 8, 768, 50257) == 50257
+    assert g2.matmul_forward_first_columns(0, 8, 768, 50257) == 0

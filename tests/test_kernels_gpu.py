@@ -384,6 +384,39 @@ def test_matmul_residual_epilogue(M, C, OC, lend, splitk_workspace):
         assert_close(out, oracle.matmul_forward(x, w, b) + r, "matmul + residual")
 
 
+# A wide product whose tiles come out just above whole rounds (the lm-head's 50257 columns at a
+# few hundred to a few thousand rows) runs as two launches over ranges of its columns, rows of
+# out staying OC floats apart: with bias, GELU, a residual, ragged rows, with and without a
+# workspace for the second launch to split K through.
+@pytest.mark.parametrize("M,C,OC,mode", [
+    (256, 256, 50257, "bias"), (1000, 256, 50257, "gelu"), (1000, 128, 50257, "resid"),
+    (2048, 128, 50257, "none"), (256, 768, 50257, "bias")])
+@pytest.mark.parametrize("lend", [False, True])
+def test_matmul_wide_product_in_two_column_ranges(M, C, OC, mode, lend, splitk_workspace):
+    ws = splitk_workspace if lend else None
+    plan = g2.matmul_forward_splitk_plan(1, M, C, OC, ws.numel() if lend else 0)
+    say(f"matmul in two column ranges M={M} C={C} OC={OC} {mode} workspace={lend} first launch {plan}")
+    first = g2.matmul_forward_first_columns(1, M, C, OC, ws.numel() if lend else 0)
+    assert 0 < first < OC and first % plan[1] == 0 and (first // plan[1]) * -(-M // plan[0]) % 256 == 0, first
+    x, w, b = mm_inputs(M, C, OC, 138, bias=mode != "none")
+    exp = oracle.matmul_forward(x, w, b)
+    full, out, pad = guard((M, OC))
+    if mode == "resid":
+        r = np.random.default_rng(139).standard_normal((M, OC), dtype=np.float32)
+        g2.matmul_forward_residual(out, dev(x), dev(w), dev(b), dev(r), 1, M, C, OC, ws)
+        exp = exp + r
+    else:
+        g2.matmul_forward_splitk(out, dev(x), dev(w), None if b is None else dev(b), 1, M, C, OC, ws,
+                                 is_gelu=mode == "gelu")
+        if mode == "gelu":
+            exp = oracle.gelu_forward(exp)
+    torch.cuda.synchronize()
+    check_guard(full, pad)
+    assert_close(out, exp, "matmul in two column ranges")
+    if lend:
+        assert int(ws[:g2.SPLITK_COUNTER_BYTES].max()) == 0, "counters not left at zero"
+
+
 def test_matmul_residual_rejects_overlap_and_null():
     M, C, OC = 64, 64, 64
     x, w, b = mm_inputs(M, C, OC, 137)
