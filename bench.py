@@ -31,7 +31,8 @@ PEAK_HBM_GBS = 8000.0           # MI355X HBM3E
 
 def dominant_traffic_bytes():
     """HBM bytes per launch of the dominant GEMM kernel (mean of the qkv, attproj and fcproj
-    shapes at M = 8192), as recorded in profiles/kernels_baseline_shapes_pmc.txt from two
+    shapes at M = 8192, the two projections with the residual add in their epilogue as the
+    driver runs them), as recorded in profiles/kernels_baseline_shapes_pmc.txt from two
     `rocprofv3 --pmc` runs of `bench.py --pmc-probe`: FETCH_SIZE (scaled x2.0: a 256 MiB copy
     reads 131 101 KiB on that counter) and WRITE_SIZE (scale 1.0).  None if the summary is
     missing or does not hold the line."""
@@ -364,6 +365,21 @@ def pmc_probe(g2):
     o = torch.empty(8, 1024, 768, device=dev)
     for _ in range(2):
         g2.attention_forward(o, None, None, qkv, 8, 1024, 768, 12)
+    del qkv, o
+    # the two projections as the driver runs them at this size (residual add in the epilogue),
+    # and the normalisation of the sum that follows them
+    for (C, OC) in ((768, 768), (3072, 768)):
+        x = torch.randn(M, C, device=dev)
+        w = torch.randn(OC, C, device=dev) * 0.02
+        r = torch.randn(M, OC, device=dev)
+        o = torch.empty(M, OC, device=dev)
+        for _ in range(2):
+            g2.matmul_forward_residual(o, x, w, None, r, 8, 1024, C, OC)
+        del x, w, o, r
+    x = torch.randn(M, 768, device=dev)
+    o = torch.empty(M, 768, device=dev)
+    dst.copy_(src)                                    # push the operands out of the caches
+    g2.layernorm_forward(o, None, None, x, torch.ones(768, device=dev), torch.zeros(768, device=dev), 8, 1024, 768)
     torch.cuda.synchronize()
     print(json.dumps({"pmc_probe": "done", "copy_bytes_each_way": src.numel() * 4}))
 
@@ -617,9 +633,11 @@ def main():
         kernels.append(row)
         log(f"  {k:26s} {prof[k]:8.3f} ms/fwd  " + (f"{row.get('TFLOP/s', 0):7.1f} TFLOP/s"
             if k in flops else f"{row.get('GB/s', 0):7.0f} GB/s"))
-    # Dominant kernel symbol: matmul_dma_kernel<128,192,4,2,false>, the instantiation that
-    # runs the qkv, attention-projection and fc-projection GEMMs (3 per layer; the fc GEMM
-    # with its GELU epilogue and the lm-head are other instantiations of the same source).
+    # Dominant kernel: matmul_dma_kernel<128,192,4,2,false>, which runs the qkv, attention-
+    # projection and fc-projection GEMMs (3 per layer; at sizes where the driver adds the residual
+    # stream in the projections' epilogues those two launches are the instantiation of the same
+    # kernel that fetches its tile of the residual during the slab loop; the fc GEMM with its
+    # GELU epilogue and the lm-head are other instantiations of the same source).
     dom = ("matmul_qkv", "matmul_attproj", "matmul_fcproj")
     dom_launches = 3 * L
     dom_flops = sum(flops[k] for k in dom) / dom_launches
@@ -631,7 +649,8 @@ def main():
                             if (args.model == "124M" and B == 8 and T == 1024) else None),
                 "traffic_source": "recorded from two rocprofv3 --pmc runs of bench.py --pmc-probe "
                                   "(profiles/kernels_baseline_shapes_pmc.txt), not counted in this run",
-                "kernel": ("matmul_dma_kernel<128,192,4,2,false>" if B * T == 8192 else
+                "kernel": ("matmul_dma_kernel<128,192,4,2,false> (qkv: plain epilogue; attproj, fcproj: "
+                           "residual add in the epilogue)" if B * T == 8192 else
                            "matmul_forward, qkv / attproj / fcproj launches (tile shape by size)"),
                 "avg_launch_ms": dom_ms, "flops_per_launch": dom_flops,
                 "launches_per_forward": dom_launches}
