@@ -1516,24 +1516,33 @@ static TileChoice choose_tile(int M, int C, int OC, bool two_largest_only, size_
   return TileChoice{best, kTileCands[best].bm, kTileCands[best].bn, tiles_of(best, M, OC), 1, best_cost};
 }
 
-// A product much wider than tall whose tiles come out just above a whole number of rounds loses
-// most of a round to the few tiles left over: the lm-head's 50257 columns are 261.75 tiles of
-// 192, so at 256 rows there are 262 tiles of 256x192 for 256 compute units, and at 1024 rows
-// 4 x 262.  Such a product is computed by two launches over ranges of its columns instead: a
-// whole number of rounds of the tile that suits it, then the few columns left with whatever
-// suits those (measured for the 768 -> 50257 lm-head: 216 -> 180 us at 256 rows, 348 -> 324 at
+// A product whose tiles come out just above a whole number of rounds loses most of a round to
+// the few tiles left over: the lm-head's 50257 columns are 261.75 tiles of 192, so at 256 rows
+// there are 262 tiles of 256x192 for 256 compute units, and at 1024 rows 4 x 262; the 2304 columns
+// of a qkv product at 1024 rows are 16 x 18 tiles of 64x128.  Such a product (1536 columns or
+// more) is computed by two launches over ranges of its columns instead: a whole number of rounds
+// of the tile that suits it, then the columns left -- at most a quarter -- with whatever suits
+// those (measured for the 768 -> 50257 lm-head: 216 -> 180 us at 256 rows, 348 -> 324 at
 // 512, 619 -> 590 at 1024, 1150 -> 1136 at 2048; within 0.5 % either way from 4096 rows on, where
-// the product is left as one launch).
+// the product is left as one launch; 768 -> 2304 at 1024 rows 40.8 -> 36.6 us; GPT-2 XL's
+// 1600 -> 6400 at 1024 / 2048 rows 188 -> 155 / 351 -> 299 us, its 1600 -> 1600 at 2048 rows,
+// which no tile of the set divides, 96 -> 85 us as one round of 128x96 over 1536 columns + 64).
 struct ColumnPlan {
   int main_cols;         // columns of the first launch; == OC: one launch
   TileChoice main, rest;
 };
 static ColumnPlan plan_columns(int M, int C, int OC, bool two_largest_only, size_t workspace_bytes) {
   ColumnPlan plan{OC, choose_tile(M, C, OC, two_largest_only, workspace_bytes), TileChoice{}};
-  if (two_largest_only || OC < 8192) return plan;
-  double best = plan.main.cost_us * 0.97;  // a second launch has to pay for itself
-  static const int kWide[] = {0, 7, 1, 8};  // 128x192, 256x192, 128x128, 256x128
+  if (two_largest_only || OC < 1536) return plan;
+  // a second launch has to pay for itself: taken only when the model puts it 3 % ahead (over M =
+  // 256 ... 8192 at the layer shapes of the four GPT-2 sizes every plan this changes got faster, by
+  // 1-17 %; taken at par or 3 % behind, as many got slower as faster)
+  double best = plan.main.cost_us * 0.97;
+  // 128x192, 256x192, 128x128, 256x128; for products of fewer than 8192 columns also 64x128,
+  // 128x96, 64x96 and 128x160
+  static const int kWide[] = {0, 7, 1, 8, 3, 2, 6, kTile128x160};
   for (int i : kWide) {
+    if ((i == 3 || i == 2 || i == 6 || i == kTile128x160) && OC >= 8192) continue;
     const long long ntm = (M + kTileCands[i].bm - 1) / kTileCands[i].bm;
     const int ntn_all = OC / kTileCands[i].bn;
     for (int ntn = ntn_all; ntn >= 1 && ntn > ntn_all - 16; ntn--) {
@@ -1542,6 +1551,7 @@ static ColumnPlan plan_columns(int M, int C, int OC, bool two_largest_only, size
       if (t > 12 * 256) break;  // the more rounds, the less the last one matters
       const int cols = ntn * kTileCands[i].bn;
       if (cols == OC) break;  // (whole rounds already)
+      if ((OC - cols) * 4 > OC) break;  // (a remainder, not a second product)
       const TileChoice rest = choose_tile(M, C, OC - cols, false, workspace_bytes);
       const double cost = tile_cost(i, t, C, 1) + rest.cost_us;
       if (cost < best) {

@@ -87,10 +87,11 @@ void matmul_forward(float* out, const float* inp, const float* weight, const flo
  * cost model so that the tiles come out in close to whole rounds over the 256 compute units
  * (the reference launches one fixed 128x128 tile shape and asserts divisibility,
  * kernels/matmul/9_matmul_async_cg_tf32_gelu.cuh:266-274).  Both are 0 for problems that
- * take another kernel (C % 32 != 0, B*T <= 16).  A product of 8192 or more columns whose tiles
- * come out just above a whole number of rounds (the lm-head at up to a few thousand rows) is
- * computed by two launches over ranges of its columns -- whole rounds of one tile, then the
- * few columns left with whatever suits those; the shape reported is the first launch's.
+ * take another kernel (C % 32 != 0, B*T <= 16).  A product of 1536 or more columns whose tiles
+ * come out just above a whole number of rounds (the lm-head at up to a few thousand rows, a
+ * 2304-wide product at 1024 rows) is computed by two launches over ranges of its columns --
+ * whole rounds of one tile, then the columns left, at most a quarter, with whatever suits
+ * those; the shape reported is the first launch's.
  * Touches no GPU. */
 int matmul_forward_tile_shape(int B, int T, int C, int OC, int* tile_rows, int* tile_cols);
 

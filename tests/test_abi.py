@@ -177,6 +177,7 @@ def test_wide_products_are_planned_as_whole_rounds_plus_the_columns_left():
         first = g2.matmul_forward_first_columns(1, M, 768, 50257)
         bm, bn = g2.matmul_forward_tile_shape(1, M, 768, 50257)
         assert 0 < first < 50257 and first % bn == 0 and (first // bn) * -(-M // bm) % 256 == 0, (M, first, bm, bn)
+    assert g2.matmul_forward_first_columns(1, 1024, 768, 2304) == 2048      # 16 x 16 tiles of 64x128, then 256 columns
     assert g2.matmul_forward_first_columns(1, 8192, 768, 50257) == 50257
     assert g2.matmul_forward_first_columns(1, 2048, 768, 3072) == 3072
     assert g2.matmul_forward_first_columns(1, 8, 768, 50257) == 50257

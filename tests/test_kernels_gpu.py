@@ -390,7 +390,8 @@ def test_matmul_residual_epilogue(M, C, OC, lend, splitk_workspace):
 # workspace for the second launch to split K through.
 @pytest.mark.parametrize("M,C,OC,mode", [
     (256, 256, 50257, "bias"), (1000, 256, 50257, "gelu"), (1000, 128, 50257, "resid"),
-    (2048, 128, 50257, "none"), (256, 768, 50257, "bias")])
+    (2048, 128, 50257, "none"), (256, 768, 50257, "bias"), (1024, 768, 2304, "bias"), (1000, 1600, 6400, "gelu"),
+    (2048, 1600, 1600, "resid")])
 @pytest.mark.parametrize("lend", [False, True])
 def test_matmul_wide_product_in_two_column_ranges(M, C, OC, mode, lend, splitk_workspace):
     ws = splitk_workspace if lend else None
