@@ -361,7 +361,10 @@ def test_matmul_llmc_signature_splits_k_through_the_thread_workspace(M, splitk_w
 @pytest.mark.parametrize("M,C,OC", [
     (8192, 768, 768), (8192, 3072, 768), (4096, 1024, 1024), (4090, 768, 770), (8192, 768, 3072),
     (6000, 768, 1536), (4096, 1280, 1280), (2048, 768, 768), (2045, 3072, 771), (256, 3072, 768),
-    (100, 96, 50), (33, 30, 17), (8, 768, 768)])
+    (100, 96, 50), (33, 30, 17), (8, 768, 768),
+    # one, two, three and five K slabs of 128x192 tiles: fewer pairs of slabs than the eight waves
+    # that take turns fetching the residual during them
+    (8192, 32, 768), (8192, 64, 768), (8192, 96, 768), (8192, 160, 768)])
 @pytest.mark.parametrize("lend", [False, True])
 def test_matmul_residual_epilogue(M, C, OC, lend, splitk_workspace):
     ws = splitk_workspace if lend else None
