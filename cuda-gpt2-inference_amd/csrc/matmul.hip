@@ -1536,7 +1536,7 @@ static ColumnPlan plan_columns(int M, int C, int OC, bool two_largest_only, size
   if (two_largest_only || OC < 1536) return plan;
   // a second launch has to pay for itself: taken only when the model puts it 3 % ahead (over M =
   // 256 ... 8192 at the layer shapes of the four GPT-2 sizes every plan this changes got faster, by
-  // 1-17 %; taken at par or 3 % behind, as many got slower as faster)
+  // 1-17 %; taken at par or 3 % behind, 19 more plans change, 12 of them for the worse)
   double best = plan.main.cost_us * 0.97;
   // 128x192, 256x192, 128x128, 256x128; for products of fewer than 8192 columns also 64x128,
   // 128x96, 64x96 and 128x160
