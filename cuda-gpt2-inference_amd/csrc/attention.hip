@@ -653,10 +653,14 @@ int attention_forward_status(float* out, float* qkvr, float* att, const float* i
     // (T / 64 sub-tiles per wave) unless several rounds of them even that out.  Below that,
     // one group per workgroup with the keys split four ways: twice the workgroups, each half as
     // long, at the price of reading every key and value twice as often and a four-way merge.
-    // Measured over T = 384 .. 1024, B = 2 .. 16, 12 and 16 heads, the four-way split wins
-    // (+2 to +19 %) up to about 1.6 T such workgroups, at most 1300, and loses 2-16 % beyond.
+    // Both forms timed over T = 256 .. 1024, B = 1 .. 16 and 12, 16, 20, 25 heads (with the first
+    // 768 workgroups dealt in alternating direction, see the kernel): the four-way split wins, by
+    // up to 40 %, below 384 / 500 / 650 / 780 workgroups of 64 queries at T = 256 / 512 / 768 /
+    // 1024 -- at T = 256 that is where its own workgroups stop being resident all at once -- and
+    // loses 3-28 % beyond; the line below is within 2.8 % of the better form at each of the 144
+    // shapes timed, 0.2 % on average.
     const long long wide = (long long)((T + 63) / 64) * B * NH;
-    const long long four_way_below = std::max<long long>(512, std::min<long long>(1300, (long long)(1.6 * T)));
+    const long long four_way_below = (long long)(0.47 * T + 265.0);
     const int P = wide < four_way_below ? 4 : 2;
     const int bq = 32 * (ATT_WAVES / P);
     const int nqb = (T + bq - 1) / bq;
