@@ -165,7 +165,8 @@ struct PhaseWeights {
   static constexpr int NIT = (NQ + 31) / 32;   // epilogue passes of 32 registers
   static constexpr int K = 256 * KG;
   f32x4 w[KG][RG];
-  f32x4 g, b;       // gamma / beta [4 * tid .. 4 * tid + 3]
+  static constexpr int GN = (K + 1023) / 1024;  // pieces of gamma / beta per thread
+  f32x4 g[GN], b[GN];  // gamma / beta [1024 p + 4 tid .. + 3]
   float bias[NIT];  // of output row 4*rg + v, for the thread that finishes register q = (rg, jg, v)
 };
 template <int ROWS, int KG, int JG, bool LN>
@@ -188,9 +189,12 @@ __device__ __forceinline__ void load_phase_weights(PhaseWeights<ROWS, KG, JG, LN
     for (int c = 0; c < KG; c++) pw.w[c][rg] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wp + c * 64));
   }
   if (LN) {
-    const int i = min(4 * tid, PW::K - 4);
-    pw.g = *reinterpret_cast<const f32x4*>(ln_w + i);
-    pw.b = *reinterpret_cast<const f32x4*>(ln_b + i);
+#pragma unroll
+    for (int p = 0; p < PW::GN; p++) {
+      const int i = min(1024 * p + 4 * tid, PW::K - 4);
+      pw.g[p] = *reinterpret_cast<const f32x4*>(ln_w + i);
+      pw.b[p] = *reinterpret_cast<const f32x4*>(ln_b + i);
+    }
   }
   const int eq = tid >> 3;
 #pragma unroll
@@ -340,9 +344,13 @@ __device__ __forceinline__ void gemm_phase(const DecodeStep& a, float* lds,
   // the last of them were still missing when the phase ended: 0.346 -> 0.337 ms per step at 8
   // sequences, 0.432 -> 0.420 at 16.)
   load_next();
-  if (LN && 4 * tid < K) {
-    *reinterpret_cast<f32x4*>(gb + 4 * tid) = pw.g;
-    *reinterpret_cast<f32x4*>(gb + K + 4 * tid) = pw.b;
+  if (LN) {
+#pragma unroll
+    for (int p = 0; p < PW::GN; p++)
+      if (1024 * p + 4 * tid < K) {
+        *reinterpret_cast<f32x4*>(gb + 1024 * p + 4 * tid) = pw.g[p];
+        *reinterpret_cast<f32x4*>(gb + K + 1024 * p + 4 * tid) = pw.b[p];
+      }
   }
   if (LN) {
     // Statistics of sequence 4*jg + r4: its row is spread over the 16 blocks of all 4 waves.
@@ -871,7 +879,13 @@ bool decode_step_supported(const GPT2Config& c, int B, int device) {
   const int C = c.channels;
   if (!device_has_grid(device)) return false;
   if (B < 1 || B > kDecodeMaxBatch || c.num_heads * 64 != C) return false;
-  if (C != 256 && C != 512 && C != 768 && C != 1024) return false;  // the instantiated sizes
+  if (B * c.num_heads > DS_GRID) return false;  // the attention phase has one workgroup per (sequence, head)
+  // the instantiated sizes (1280 channels, GPT-2 large: with 9 to 16 sequences the fcproj phase's 20
+  // weight pieces and 20 activation pieces per group of four sequences no longer all fit in
+  // registers and 80-420 bytes per lane spill; a step is still a third shorter than one launch per
+  // operation: 1.79 / 1.83 against 2.74 / 2.89 ms at 9 / 12 sequences, 36 layers; its 20 heads allow
+  // 12 sequences)
+  if (C != 256 && C != 512 && C != 768 && C != 1024 && C != 1280) return false;
   return decode_step_lds_bytes(c, B, c.max_seq_len - 1) <= 160 * 1024;
 }
 
@@ -893,12 +907,13 @@ int decode_step_launch(const DecodeStep& step, const GPT2Config& c, int device) 
   const void* kernel = kg1 == 1   ? kernel_for<1, 8>(jg)
                        : kg1 == 2 ? kernel_for<2, 16>(jg)
                        : kg1 == 3 ? kernel_for<3, 24>(jg)
-                                  : kernel_for<4, 16>(jg);
+                       : kg1 == 4 ? kernel_for<4, 16>(jg)
+                                  : kernel_for<5, 10>(jg);
   // the dynamic-LDS limit is a per-device property of the kernel: remembered per thread and
   // device, like the GEMM launchers do
   if (lds > 48 * 1024) {
     static thread_local int raised_on = -1;
-    static thread_local bool raised[4][4];
+    static thread_local bool raised[5][4];
     if (raised_on != device) {
       raised_on = device;
       for (auto& row : raised)

@@ -390,6 +390,15 @@ def test_gpt2_prefill_and_decode_match_the_full_forward(cfg, B, T0, steps):
     (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=16, channels=1024), 9, 30, 3),
     (dict(max_seq_len=48, vocab_size=1031, num_layers=2, num_heads=12, channels=768), 17, 20, 3),
     (dict(max_seq_len=48, vocab_size=331, num_layers=2, num_heads=12, channels=768), 64, 30, 3),
+    # GPT-2 large's width (1280 channels, 20 heads): one to four groups of four sequences, ranges of
+    # positions at a long context
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=20, channels=1280), 3, 20, 3),
+    (dict(max_seq_len=64, vocab_size=1031, num_layers=3, num_heads=20, channels=1280), 8, 30, 4),
+    (dict(max_seq_len=400, vocab_size=331, num_layers=2, num_heads=20, channels=1280), 2, 390, 3),
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=20, channels=1280), 9, 20, 2),
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=20, channels=1280), 12, 25, 3),
+    # (13 sequences of 20 heads are more (sequence, head) pairs than the kernel has workgroups)
+    (dict(max_seq_len=64, vocab_size=331, num_layers=2, num_heads=20, channels=1280), 13, 25, 2),
 ])
 def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_path(cfg, B, T0, steps):
     print(f"persistent decode cfg={cfg} B={B} T0={T0} steps={steps}", flush=True)
@@ -407,7 +416,7 @@ def test_gpt2_persistent_decode_matches_the_oracle_and_the_launch_per_operation_
             model.decode_options(persistent=persistent)
             model.prefill(dids[:, :T0].contiguous())
             # the path that is meant runs: the persistent kernel takes up to 16 sequences
-            assert (model.decode_probe_size() > 0) == (persistent and B <= 16)
+            assert (model.decode_probe_size() > 0) == (persistent and B <= 16 and B * cfg["num_heads"] <= 256)
             out = []
             for s in range(steps):
                 print(f"  persistent={persistent} step {s}", flush=True)
