@@ -1831,8 +1831,10 @@ int matmul_forward_residual_status(float* out, const float* inp, const float* we
   using namespace g2;
   if (!resid) return fail(GPT2HIP_EINVAL, "matmul_forward_residual: null residual");
   // the kernels read resid and write out through pointers they are told do not alias
-  const long long n = (long long)(B > 0 ? B : 0) * (T > 0 ? T : 0) * (OC > 0 ? OC : 0);
-  if (out && out < resid + n && resid < out + n)
+  const unsigned long long bytes =
+      (unsigned long long)(B > 0 ? B : 0) * (unsigned long long)(T > 0 ? T : 0) * (OC > 0 ? OC : 0) * sizeof(float);
+  const uintptr_t o = reinterpret_cast<uintptr_t>(out), r = reinterpret_cast<uintptr_t>(resid);
+  if (out && o < r + bytes && r < o + bytes)
     return fail(GPT2HIP_EINVAL, "matmul_forward_residual: out and resid overlap");
   return matmul_dispatch(out, inp, weight, bias, B, T, C, OC, false, nullptr, nullptr, workspace,
                          workspace_bytes, nullptr, resid);
