@@ -259,16 +259,21 @@ static int launch_layernorm(float* res_out, float* out, float* mean, float* rstd
   //             2048: 5.5 / 5.3 / 7.2 / 9.9;  1024: 3.7 / 4.3 / 6.6 / 9.3
   //   C = 1024: N = 8192: 24.3 / 23.6 / 22.3 / 21.5;  4096: 14.0 / 11.6 / 12.4 / 14.4;
   //             2048: 7.5 / 6.4 / 7.6 / 13.4;  1024: 4.9 / 5.0 / 6.8 / 12.3
-  // (eight rows at N = 4096 are 128 workgroups: half the chip idle).
+  // (eight rows at N = 4096 are 128 workgroups: half the chip idle).  The plain form takes two rows
+  // per wave from 4096 rows on and one below, always without bounds checks where C is a multiple of
+  // 256 and N of 8 (one row with bounds checks had been the form below 4096 rows: 6.9 -> 5.3 us at
+  // 3072 x 1024, 6.3 -> 5.5 at 2048 x 1280).
   const bool wide = N >= 4096;
 #define G2_LN(NV, ROWS, EXACT, NTS, ...)                                                        \
   hipLaunchKernelGGL((layernorm_rows_kernel<NV, ROWS, FUSED, EXACT, NTS, ##__VA_ARGS__>),       \
                      dim3((N + kWavesPerBlock * ROWS - 1) / (kWavesPerBlock * ROWS)), block, 0, stream(), \
                      res_out, out, mean, rstd, inp1, inp2, weight, bias, N, C)
 #define G2_LN_ROWS(NV)                                              \
-  if (C == 256 * NV && N % 8 == 0 && (long long)N * C * 4 < (1LL << 31) && (FUSED || wide)) { \
-    if (!FUSED) {                                                   \
+  if (C == 256 * NV && N % 8 == 0 && (long long)N * C * 4 < (1LL << 31)) { \
+    if (!FUSED && wide) {                                           \
       G2_LN(NV, 2, true, true);                                     \
+    } else if (!FUSED) {                                            \
+      G2_LN(NV, 1, true, true);                                     \
     } else if (NV == 4 && N >= 8192) {                              \
       G2_LN(NV, 8, true, false);                                    \
     } else if (N >= 8192) {                                         \
