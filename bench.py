@@ -502,7 +502,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--model", choices=("124M", "350M"), default="124M")
+    ap.add_argument("--model", choices=("124M", "350M", "774M", "1558M"), default="124M",
+                    help="124M is the benchmark's model; the others are the wider GPT-2 sizes (with --batch)")
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--seq-len", type=int, default=1024)
     ap.add_argument("--no-standalone", action="store_true")
@@ -539,7 +540,7 @@ def main():
     if args.clock_probe:
         clock_probe(g2)
         return
-    cfg = dict(g2.GPT2_124M if args.model == "124M" else g2.GPT2_350M)
+    cfg = dict({"124M": g2.GPT2_124M, "350M": g2.GPT2_350M, "774M": g2.GPT2_774M, "1558M": g2.GPT2_1558M}[args.model])
     B = args.batch or (8 if args.model == "124M" else 4)
     T = args.seq_len
     model = g2.GPT2(**cfg)

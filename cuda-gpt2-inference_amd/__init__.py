@@ -104,6 +104,8 @@ PROF_CATEGORIES = ("encoder", "layernorm", "matmul_qkv", "attention", "matmul_at
 
 GPT2_124M = dict(max_seq_len=1024, vocab_size=50257, num_layers=12, num_heads=12, channels=768)
 GPT2_350M = dict(max_seq_len=1024, vocab_size=50257, num_layers=24, num_heads=16, channels=1024)
+GPT2_774M = dict(max_seq_len=1024, vocab_size=50257, num_layers=36, num_heads=20, channels=1280)    # "large"
+GPT2_1558M = dict(max_seq_len=1024, vocab_size=50257, num_layers=48, num_heads=25, channels=1600)   # "XL"
 
 _lib: Optional[ctypes.CDLL] = None
 
